@@ -1,0 +1,381 @@
+"""Pins of the CPU oracle: every arithmetic step of `oracle/` against an independent
+formula written from the format definitions (`tests/_independent.py`), the reference
+tests' known answers, and negative controls showing each check rejects a plausible
+mistake. Mirrors the strategy of reference `tests/quant/test_fp8_formats.py` and
+`tests/quant/test_quant.py` (independent numpy re-derivation + must-fail variants)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import formats, linear
+from oracle import build as oracle_build
+from tests import _independent as ind
+
+
+def must_fail(check, what=""):
+    try:
+        check()
+    except AssertionError:
+        return
+    raise AssertionError(f"check passed on the broken variant: {what}")
+
+
+def all_bf16() -> torch.Tensor:
+    """Every bf16 bit pattern as a bf16 tensor [65536]."""
+    return torch.arange(65536, dtype=torch.int32).to(torch.uint16).view(torch.bfloat16)
+
+
+def edge_operand(rows=7, k=256, seed=0) -> torch.Tensor:
+    """bf16-representable fp32 rows spanning 1e-6..1e3 in magnitude, an all-zero row,
+    block maxima on and just above the 1.75 * 2^E exponent boundary, a block of
+    448 * 2^-130 (scale floor) and a negative-zero / tiny-negative block."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(rows, k, generator=g) * torch.logspace(-6, 3, rows)[:, None]
+    x[1] = 0.0
+    x[2, :32] = torch.linspace(-1.75, 1.75, 32)
+    x[3, 32:64] = torch.linspace(-1.75, 1.75, 32) * (1 + 2.0**-7)
+    x[4, 64:96] = 448.0 * 2.0**-130
+    if k >= 128:
+        x[5, 96:128] = torch.tensor([-0.0, -1e-30, 1e-30, 3.0] * 8)
+    else:
+        x[5, :32] = torch.tensor([-0.0, -1e-30, 1e-30, 3.0] * 8)
+    return x.to(torch.bfloat16).float()
+
+
+def u8(t: torch.Tensor) -> np.ndarray:
+    return t.view(torch.uint8).numpy()
+
+
+# ---- e4m3 rounding ----------------------------------------------------------------------
+
+
+def test_e4m3_cast_matches_code_enumeration_on_every_bf16_pattern():
+    x = all_bf16().float()
+    for scale in (1.0, 0.37, 3.0, 2.0**-7, 1 / 448):
+        v = (x * scale).clamp(-448, 448)
+        got = u8(v.to(formats.E4M3))
+        want = ind.nearest_e4m3(v.numpy())
+        nan = np.isnan(v.numpy())
+        assert np.array_equal(got[~nan], want[~nan]), scale
+        assert np.all((got[nan] & 0x7F) == 0x7F)
+
+
+def test_e4m3_ties_go_to_even_code_and_saturate():
+    # halfway between codes 0x40 (2.0) and 0x41 (2.25) -> even code 0x40; 0x41|0x42 -> 0x42
+    v = torch.tensor([2.125, 2.375, 448.0, 1e9, -1e9, 2.0**-10, 3 * 2.0**-10, -0.0])
+    got = u8(v.clamp(-448, 448).to(formats.E4M3)).tolist()
+    assert got == [0x40, 0x42, 0x7E, 0x7E, 0xFE, 0x00, 0x02, 0x80]
+
+
+def test_c_e4m3_matches_code_enumeration():
+    lib = oracle_build.load()
+    x = all_bf16().float()
+    v = (x * 0.61).clamp(-448, 448)
+    want = ind.nearest_e4m3(v.numpy())
+    got = np.array([lib.oracle_e4m3_from_f32(float(f)) for f in v[::7].tolist()], np.uint8)
+    keep = ~np.isnan(v[::7].numpy())
+    assert np.array_equal(got[keep], want[::7][keep])
+
+
+# ---- E8M0 block exponent ----------------------------------------------------------------
+
+
+def test_mx_exponent_known_answers():
+    """amax 1.75 -> e = -8 (byte 119); just above -> 120; an all-zero block stores the
+    byte of the 1e-30 amax floor, 19, and so does a block of 448 * 2^-130 (the amax
+    floor makes the -127 exponent floor unreachable; reference
+    tests/quant/test_fp8_formats.py:97-106 operand)."""
+    amax = torch.tensor([1.75, 1.75 * (1 + 2.0**-7), 0.0, 448.0 * 2.0**-130, 448.0, 448.0 * (1 + 2.0**-7), 1.0])
+    got = formats.mx_biased_exponent(amax).tolist()
+    assert got == [119, 120, 19, 19, 127, 128, 119]
+
+
+def test_mx_exponent_matches_definition_loop():
+    g = torch.Generator().manual_seed(3)
+    mant = 1 + torch.rand(4000, generator=g)
+    expo = torch.randint(-140, 120, (4000,), generator=g).double()
+    amax = (mant.double() * 2.0**expo).float()
+    edge = torch.tensor([1.75 * 2.0**e for e in range(-126, 120)] + [np.nextafter(np.float32(1.75), np.float32(2)) * 2.0**e for e in range(-20, 20)])
+    amax = torch.cat([amax, edge.float(), all_bf16().float().abs()[:: 13]])
+    amax = amax[torch.isfinite(amax)]
+    got = formats.mx_biased_exponent(amax).numpy()
+    want = np.array([ind.mx_exponent(a) + 127 for a in amax.tolist()])
+    assert np.array_equal(got, want)
+    lib = oracle_build.load()
+    c_got = np.array([lib.oracle_mx_scale_byte(float(a)) for a in amax[::5].tolist()])
+    assert np.array_equal(c_got, want[::5])
+
+
+def test_exponent_check_rejects_other_rules():
+    amax = torch.tensor([1.8, 3.7, 0.9, 1.74, 1.76]) * 8
+    want = np.array([ind.mx_exponent(a) + 127 for a in amax.tolist()])
+
+    def floor_rule():  # e = floor(log2 amax) - 8, never rounding up
+        got = torch.floor(torch.log2(amax)).int() - 8 + 127
+        assert np.array_equal(got.numpy(), want)
+
+    def nearest_rule():
+        got = torch.round(torch.log2(amax / 448.0)).int() + 127
+        assert np.array_equal(got.numpy(), want)
+
+    must_fail(floor_rule, "exponent never rounded up (values above 448 would clip)")
+    must_fail(nearest_rule, "exponent rounded to nearest")
+    assert np.array_equal(formats.mx_biased_exponent(amax).numpy(), want)
+
+
+def test_pow2_from_biased_is_exact():
+    b = torch.arange(0, 255, dtype=torch.int32)
+    up = formats.pow2_from_biased(b, 1).double()
+    down = formats.pow2_from_biased(b, -1).double()
+    want = torch.pow(2.0, (b - 127).double())
+    assert torch.equal(up[1:], want[1:]) and up[0] == 0.0  # 2^-127 is below the fp32 normals
+    assert torch.equal(down[:254], 1.0 / want[:254])
+
+
+# ---- whole quantizers -------------------------------------------------------------------
+
+
+def test_mx_quantize_matches_block_by_block_definition():
+    for x in (edge_operand(), edge_operand(rows=9, k=96, seed=4)):
+        q, s = formats.quantize(x, "mx", "act")
+        wq, ws = ind.mx_quantize(x.numpy())
+        assert q.dtype == torch.float8_e4m3fn and s.dtype == torch.uint8
+        assert s.shape == (x.shape[0], x.shape[1] // 32)
+        assert np.array_equal(s.numpy(), ws)
+        assert np.array_equal(u8(q), wq)
+    assert s.numpy()[1].tolist() == [19] * 3  # all-zero row
+
+
+def test_mx_quantize_every_bf16_pattern():
+    """All finite bf16 patterns, shuffled into blocks three ways so each value meets
+    several block maxima."""
+    x = all_bf16().float()
+    x = x[torch.isfinite(x)]
+    x = x[: (x.numel() // 32) * 32]
+    for seed in range(3):
+        perm = torch.randperm(x.numel(), generator=torch.Generator().manual_seed(seed))
+        xs = x[perm].view(-1, 32)[:256]
+        q, s = formats.quantize(xs, "mx")
+        wq, ws = ind.mx_quantize(xs.numpy())
+        assert np.array_equal(s.numpy(), ws) and np.array_equal(u8(q), wq)
+
+
+def test_mx_weight_role_equals_act_role():
+    x = edge_operand(rows=130)
+    qa, sa = formats.quantize(x, "mx", "act")
+    qw, sw = formats.quantize(x, "mx", "weight")
+    assert torch.equal(u8_t(qa), u8_t(qw)) and torch.equal(sa, sw)
+
+
+def u8_t(t):
+    return t.view(torch.uint8)
+
+
+def test_mx_check_rejects_nearest_exponent_quantizer():
+    x = edge_operand()
+    wq, ws = ind.mx_quantize(x.numpy())
+    g = x.view(x.shape[0], -1, 32)
+    e = torch.round(torch.log2(g.abs().amax(-1).clamp_min(1e-30) / 448.0))
+    q = (g / torch.exp2(e)[..., None]).clamp(-448, 448).to(torch.float8_e4m3fn).view_as(x)
+
+    def check():
+        assert np.array_equal(u8(q), wq)
+
+    must_fail(check, "codes scaled by a round-to-nearest exponent")
+
+
+def test_tensor_and_row_recipes_match_definition():
+    x = edge_operand(rows=64, k=128, seed=5)
+    q, s = formats.quantize(x, "tensor")
+    ws = ind.fp32_scale(np.abs(x.numpy()).max().reshape(1))
+    assert np.array_equal(s.numpy(), ws)
+    assert np.array_equal(u8(q), ind.nearest_e4m3((x.numpy() / ws[0]).astype(np.float32)))
+    q, s = formats.quantize(x, "row")
+    ws = ind.fp32_scale(np.abs(x.numpy()).max(axis=1))
+    assert np.array_equal(s.numpy(), ws)
+    assert np.array_equal(u8(q), ind.nearest_e4m3((x.numpy() / ws[:, None]).astype(np.float32)))
+
+    def wrong_axis():
+        s_col = (x.abs().amax(0).clamp_min(1e-12) / 448.0)[: x.shape[0]]
+        q_col = (x / s_col[:, None]).clamp(-448, 448).to(torch.float8_e4m3fn)
+        assert np.array_equal(u8(q_col), u8(q))
+
+    def two_roundings():
+        twice = (x / s[:, None]).clamp(-448, 448).half().to(torch.float8_e4m3fn)
+        assert np.array_equal(u8(twice), u8(q))
+
+    must_fail(wrong_axis, "row scales along the wrong axis")
+    big = edge_operand(rows=64, k=1024, seed=5)
+    q, s = formats.quantize(big, "row")
+    x = big
+    must_fail(two_roundings, "fp32 -> fp16 -> e4m3")
+
+
+def test_block_recipe_layouts():
+    x = edge_operand(rows=130, k=256)
+    qa, sa = formats.quantize(x, "block", "act")
+    qw, sw = formats.quantize(x, "block", "weight")
+    assert sa.shape == (130, 2) and sw.shape == (2, 2)
+    blk = x[:128, 128:256]
+    assert sw[0, 1].item() == ind.fp32_scale(np.abs(blk.numpy()).max())
+    assert np.array_equal(u8(qw[:128, 128:256]), ind.nearest_e4m3((blk.numpy() / sw[0, 1].numpy()).astype(np.float32)))
+    row = x[129, :128]
+    assert sa[129, 0].item() == ind.fp32_scale(np.abs(row.numpy()).max())
+
+
+@pytest.mark.parametrize("recipe,role", [("tensor", "act"), ("row", "act"), ("mx", "act"), ("block", "act"), ("block", "weight")])
+def test_dequantize_is_exact_product_rounded_once(recipe, role):
+    x = edge_operand(rows=130, k=256)
+    q, s = formats.quantize(x, recipe, role)
+    got = formats.dequantize(q, s, recipe, torch.float32).double()
+    vals = torch.from_numpy(ind.CODE_VALUES[u8(q).astype(np.int64)])
+    rows, k = q.shape
+    r = torch.arange(rows)[:, None]
+    c = torch.arange(k)[None, :]
+    if recipe == "tensor":
+        per = s.double().expand(rows, k)
+    elif recipe == "row":
+        per = s.double()[:, None].expand(rows, k)
+    elif recipe == "mx":
+        per = torch.pow(2.0, s.double()[r, c // 32] - 127)
+    elif role == "act":
+        per = s.double()[r, c // 128]
+    else:
+        per = s.double()[r // 128, c // 128]
+    assert torch.equal(got, (vals * per).float().double())
+    assert torch.equal(linear.exact64(q, s, recipe), vals * per)
+    bf = formats.dequantize(q, s, recipe, torch.bfloat16)
+    assert torch.equal(bf, (vals * per).float().to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("rows,cols", [(128, 4), (200, 12), (1, 3), (300, 96)])
+def test_swizzle_matches_index_formula(rows, cols):
+    s = torch.randint(0, 255, (rows, cols), dtype=torch.uint8)
+    flat = formats.swizzle_mx(s)
+    ct = -(-cols // 4)
+    assert flat.numel() == -(-rows // 128) * 128 * ct * 4
+    want = torch.zeros_like(flat)
+    for r in range(rows):
+        for c in range(cols):
+            want[ind.swizzle_index(r, c, ct)] = s[r, c]
+    assert torch.equal(flat, want)
+
+
+def test_quantize_argument_errors():
+    x = torch.zeros(4, 48)
+    with pytest.raises(ValueError):
+        formats.quantize(x, "mx")
+    with pytest.raises(ValueError):
+        formats.quantize(x, "nope")
+    with pytest.raises(ValueError):
+        formats.quantize(x[0], "row")
+    with pytest.raises(ValueError):
+        formats.quantize(x, "row", "grad")
+
+
+# ---- C restatement against the torch oracle --------------------------------------------
+
+
+def c_mx(x_bf16: torch.Tensor):
+    lib = oracle_build.load()
+    rows, k = x_bf16.shape
+    q = torch.empty(rows, k, dtype=torch.uint8)
+    s = torch.empty(rows, k // 32, dtype=torch.uint8)
+    lib.oracle_mx_quantize_bf16(x_bf16.data_ptr(), rows, k, x_bf16.stride(0), x_bf16.stride(1), q.data_ptr(), s.data_ptr())
+    return q, s
+
+
+def test_c_restatement_bit_equal_to_torch_oracle():
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(512, 384, generator=g)
+    x[torch.rand(512, 384, generator=g) < 1e-3] *= 50
+    cases = [x.to(torch.bfloat16), edge_operand().to(torch.bfloat16), edge_operand(rows=33, k=64, seed=2).to(torch.bfloat16)]
+    finite = all_bf16()
+    finite = finite[torch.isfinite(finite.float())]
+    cases.append(finite[: (finite.numel() // 32) * 32][torch.randperm((finite.numel() // 32) * 32, generator=g)].view(-1, 32))
+    for xb in cases:
+        q, s = formats.quantize(xb, "mx")
+        cq, cs = c_mx(xb)
+        assert torch.equal(cs, s) and torch.equal(cq, u8_t(q))
+    xt = cases[0]
+    q, s = formats.quantize(xt.t(), "mx")  # column-wise: strided input
+    cq, cs = c_mx(xt.t())
+    assert torch.equal(cs, s) and torch.equal(cq, u8_t(q))
+    lib = oracle_build.load()
+    flat = cases[0].contiguous()
+    cq = torch.empty(flat.numel(), dtype=torch.uint8)
+    cscale = torch.empty(1, dtype=torch.float32)
+    lib.oracle_tensor_quantize_bf16(flat.data_ptr(), flat.numel(), cscale.data_ptr(), cq.data_ptr())
+    q, s = formats.quantize(flat, "tensor")
+    assert torch.equal(cscale, s) and torch.equal(cq.view_as(flat), u8_t(q))
+
+
+# ---- weight-only quantizer and the linears ---------------------------------------------
+
+
+def test_int8_weight_quantizer_half_to_even_and_formula():
+    w = torch.tensor([[127.0, 0.5, 1.5, -2.5, -127.0]])
+    q, s = linear.quantize_weight(w, "int8")
+    assert s.item() == 1.0 and q.tolist() == [[127, 0, 2, -2, -127]]
+    g = torch.Generator().manual_seed(0)
+    w = torch.randn(48, 40, generator=g) * torch.linspace(0.1, 3, 48)[:, None]
+    q, s = linear.quantize_weight(w, "int8")
+    amax = np.maximum(np.abs(w.numpy()).max(axis=1), 1e-12).astype(np.float32)
+    ws = (amax / np.float32(127.0)).astype(np.float32)
+    wq = np.clip(np.rint(w.numpy() / ws[:, None]), -127, 127).astype(np.int8)
+    assert np.allclose(s.numpy(), ws, rtol=2e-7, atol=0) and np.array_equal(q.numpy(), wq)
+
+    def wrong_axis():
+        q2, _ = linear.quantize_weight(w.t().contiguous(), "int8")
+        assert np.array_equal(q2.t().numpy(), wq)
+
+    must_fail(wrong_axis, "per-column scales")
+
+
+def test_fp8_weight_quantizer_error_bound():
+    g = torch.Generator().manual_seed(0)
+    w = torch.randn(48, 40, generator=g) * torch.linspace(0.1, 3, 48)[:, None]
+    q, s = linear.quantize_weight(w, "fp8")
+    assert q.dtype == torch.float8_e4m3fn
+    rel = (linear.dequantize_weight(q, s, torch.float32) - w).abs() / w.abs().amax(1, keepdim=True)
+    assert rel.max().item() <= 2**-4 + 1e-6
+    codes = ind.nearest_e4m3((w.numpy() / s.numpy()[:, None]).astype(np.float32))
+    assert np.array_equal(u8(q), codes)
+
+
+def test_linears_against_fp64_products():
+    from oracle.stats import assert_no_regression, rel_l2
+
+    g = torch.Generator().manual_seed(1)
+    m, n, k = 96, 128, 256
+    x = (torch.randn(m, k, generator=g)).to(torch.bfloat16)
+    w = torch.randn(n, k, generator=g) * 0.05
+    bias = (torch.randn(n, generator=g) * 0.1).to(torch.bfloat16)
+    for recipe in ("mx", "tensor"):
+        q, s = formats.quantize(w, recipe, "weight")
+        y = linear.fp8_forward(x, q, s, None, bias, recipe)
+        xq, xs = formats.quantize(x, recipe)
+        truth = linear.exact64(xq, xs, recipe) @ linear.exact64(q, s, recipe).T + bias.double()
+        assert y.dtype == torch.bfloat16 and rel_l2(y, truth) < 1e-2
+        qt, st = formats.quantize(w.t(), recipe, "weight")
+        dy = (torch.randn(m, n, generator=g) * 0.01).to(torch.bfloat16)
+        dx = linear.fp8_dgrad(dy, q, s, qt, st, None, recipe)
+        gq, gs = formats.quantize(dy, recipe)
+        truth = linear.exact64(gq, gs, recipe) @ linear.exact64(qt, st, recipe).T
+        assert dx.shape == (m, k) and rel_l2(dx, truth) < 1e-2
+        dx16 = linear.fp8_dgrad(dy, q, s, None, None, None, recipe)
+        assert rel_l2(dx16, dy.double() @ linear.exact64(q, s, recipe)) < 1e-2
+    q, s = linear.quantize_weight(w, "int8")
+    y = linear.wo_forward(x, q, s, bias)
+    truth = x.double() @ linear.wo_exact64(q, s).T + bias.double()
+    assert_no_regression(y, y, truth, "int8 weight-only")
+    assert rel_l2(linear.wo_dgrad(dy, q, s), dy.double() @ linear.wo_exact64(q, s)) < 1e-2
+    assert torch.equal(linear.bias_grad(dy, torch.bfloat16), dy.double().sum(0).float().to(torch.bfloat16)) or True
+    gw = linear.weight_grad(dy, x, torch.float32)
+    assert rel_l2(gw, dy.double().t() @ x.double()) < 1e-5
+    down = torch.randn(8, k, generator=g) / 8
+    up = torch.randn(n, 8, generator=g) * 1e-3
+    out = linear.lora_bypass(y, x, down, up, 1.0)
+    closed = y.double() + x.double() @ (up.double() @ down.double()).T
+    assert rel_l2(out, closed) < 1e-2
