@@ -1,0 +1,105 @@
+/* C ABI of the MI355X (gfx950) quantized-linear kernels.
+ *
+ * The reference (KohakuMossTrainer, pure Python) has no FFI of its own: its backends are
+ * Python modules that register a launcher pair per op
+ *     register_launchers(backend, fwd, dgrad)      src/kohakumoss_kernels/fp8/op.py:43-46
+ *                                                  src/kohakumoss_kernels/quant/__init__.py:66-68
+ * and the Triton backend's launchers call JIT kernels. This library is what a "hip"
+ * backend's launchers call instead, through ctypes. Every entry point
+ *   - takes plain device pointers, sizes and a hipStream_t (as void*; NULL = the null stream),
+ *   - launches asynchronously on that stream, never synchronizes, never allocates,
+ *   - never writes its inputs,
+ *   - returns KM_OK or a negative error code; km_last_error() then describes it
+ *     (thread local). The Python side turns a non-zero code into RuntimeError, the
+ *     reference's "cannot build / launch here" class (src/kohakumoss_kernels/errors.py:12-17).
+ */
+#ifndef KM_KERNELS_H
+#define KM_KERNELS_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { KM_OK = 0, KM_ERR_ARG = -1, KM_ERR_LAUNCH = -2, KM_ERR_UNSUPPORTED = -3 };
+enum { KM_BF16 = 0, KM_F16 = 1, KM_F32 = 2 };          /* 16-bit activation / output dtypes */
+enum { KM_Q_INT8 = 0, KM_Q_E4M3 = 1 };                  /* weight-only code formats */
+enum { KM_SCALES_ROWMAJOR = 0, KM_SCALES_PACKED = 1 };  /* MX scale layouts the GEMM reads */
+enum { KM_KERNEL_GEMM_MX = 0, KM_KERNEL_GEMM_FP8 = 1, KM_KERNEL_WO_FWD = 2, KM_KERNEL_WO_DGRAD = 3 };
+
+int km_abi_version(void);
+const char *km_last_error(void);
+
+/* MXFP8 quantizer of a logical [rows, cols] operand whose element (r, c) is at
+ * x[r*stride_row + c*stride_col] (strides in elements; dtype KM_BF16 / KM_F16). Blocks of 32
+ * run along cols (cols % 32 == 0). Writes q [rows, cols] e4m3fn bytes and the biased E8M0 scale
+ * bytes in up to two layouts (either pointer may be NULL, not both): `scales` [rows, cols/32]
+ * dense row-major (the reference's layout) and `scales_packed`, the MFMA-packed copy
+ * km_gemm_mx reads fastest (cols % 128 == 0; km_scales_packed_bytes() bytes, the caller zero-
+ * fills it first when rows % 128 != 0). A transposed view (stride_row == 1) is the reference's
+ * column-wise quantization quantize(x.t(), "mx").
+ * Replaces fp8.formats.quantize(x, "mx", role) (src/kohakumoss_kernels/fp8/formats.py:94-99),
+ * Triton quantize_blocks(x, mx=True) (backends/triton/fp8/quantize.py:171-187) and, for the
+ * packed output, Triton quantize_mx_swizzled (backends/triton/fp8/quantize.py:190-198). */
+int km_quant_mx(const void *x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,
+                int dtype, void *q, void *scales, void *scales_packed, void *stream);
+
+/* MFMA-packed copy of an MX scale matrix. For every K step of 128 columns and group of 128
+ * rows it holds 512 bytes ordered [row % 16][block % 4][(row % 128) / 16]: byte (r, b) of the
+ * natural [rows, cols/32] matrix sits at
+ *   ((((b/4) * ceil(rows/128) + r/128) * 16 + r%16) * 4 + b%4) * 8 + (r%128)/16.
+ * A lane of the block-scaled MFMA then finds the scales of the eight 16-row tiles of its
+ * wavefront in 8 consecutive bytes and a wavefront reads them with one 512-byte load. It plays
+ * the role of the vendor swizzle the reference keeps in `aux`
+ * (swizzle_mx, src/kohakumoss_kernels/fp8/formats.py:128-136). Rows past `rows` are padding. */
+int64_t km_scales_packed_bytes(int64_t rows, int64_t cols);
+int km_scales_pack(const void *scales, int64_t rows, int64_t cols, void *out, void *stream);
+
+/* Per-tensor e4m3 quantizer: *scale_out = max(amax, 1e-12) / 448 (IEEE division),
+ * q = e4m3(clamp(x / scale)). amax_workspace is 4 bytes of device memory the call owns
+ * while it runs. Replaces fp8.formats.quantize(x, "tensor")
+ * (src/kohakumoss_kernels/fp8/formats.py:77-79) and Triton quantize_tensor
+ * (backends/triton/fp8/quantize.py:161-168). */
+int km_quant_tensor(const void *x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,
+                    int dtype, void *q, float *scale_out, uint32_t *amax_workspace, void *stream);
+
+/* C[M,N] = (A .* 2^(a_scale-127)) (B .* 2^(b_scale-127))^T + bias, A [M,K] and B [N,K] e4m3fn
+ * row-major (K contiguous), scales E8M0 bytes, both in the layout scale_layout names
+ * (KM_SCALES_ROWMAJOR: [M,K/32] / [N,K/32]; KM_SCALES_PACKED: see km_scales_pack), fp32 accumulation
+ * over all of K on the block-scaled MFMA, bias [N] (out_dtype, may be NULL) added in fp32, one
+ * rounding to out_dtype. K % 128 == 0. config selects a tile configuration
+ * (0 <= config < km_num_configs(KM_KERNEL_GEMM_MX)).
+ * Replaces Triton dot_scaled_mm / promote_mm (backends/triton/fp8/gemm.py:108-171,219-231). */
+int km_gemm_mx(const void *a, const void *a_scale, const void *b, const void *b_scale,
+               const void *bias, void *c, int64_t M, int64_t N, int64_t K, int out_dtype,
+               int scale_layout, int config, void *stream);
+
+/* Per-tensor fp8 GEMM: C = (A B^T) * (*sa * *sb) + bias, sa / sb device fp32 scalars.
+ * Replaces Triton scaled_mm for the tensor recipe (backends/triton/fp8/gemm.py:66-105,187-202)
+ * and torch._scaled_mm (backends/triton/fp8/linear.py:121-130). K % 128 == 0. */
+int km_gemm_fp8_tensor(const void *a, const float *sa, const void *b, const float *sb,
+                       const void *bias, void *c, int64_t M, int64_t N, int64_t K, int out_dtype,
+                       int config, void *stream);
+
+/* Weight-only forward: y[M,N] = (x[M,K] @ q[N,K]^T) * scale[N] + bias[N]; q int8 or e4m3fn
+ * widened exactly to the activation dtype in registers, fp32 accumulation, scale and bias on
+ * the accumulator, one rounding. Replaces Triton _fwd_kernel (backends/triton/quant.py:27-77). */
+int km_wo_gemm_fwd(const void *x, const void *q, const float *scale, const void *bias, void *y,
+                   int64_t M, int64_t N, int64_t K, int q_format, int dtype, int config,
+                   void *stream);
+
+/* Weight-only input gradient: dx[M,K] = dy[M,N] @ round_dtype(q[N,K] * scale[N]); the scaled
+ * weight tile is rounded once to the activation dtype, as dequantize-then-matmul does.
+ * Replaces Triton _dgrad_kernel (backends/triton/quant.py:80-129). */
+int km_wo_gemm_dgrad(const void *dy, const void *q, const float *scale, void *dx, int64_t M,
+                     int64_t N, int64_t K, int q_format, int dtype, int config, void *stream);
+
+/* Tile configurations per kernel, for the host-side tuning table (the reference enumerates its
+ * Triton tiles in backends/triton/fp8/linear.py:39-75 and backends/triton/quant.py:132-141). */
+int km_num_configs(int kernel);
+int km_config_desc(int kernel, int config, char *buf, int len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,503 @@
+// fp8 GEMMs for gfx950 on the block-scaled MFMA (V_MFMA_SCALE_F32_16X16X128_F8F6F4):
+//
+//   C[M,N] = A[M,K] B[N,K]^T (+ bias), A and B e4m3fn with K contiguous, fp32 accumulation
+//   over all of K, scales applied in fp32 by the MFMA (mx) or on the accumulator (tensor),
+//   bias added in fp32, one rounding at the store.
+//
+// Replaces the reference's Triton GEMMs (src/kohakumoss_kernels/backends/triton/fp8/gemm.py:
+// _dot_scaled_kernel :137-171 and _promote_kernel :108-134 for mx, _scaled_kernel :66-105 for
+// the per-tensor recipe; the shared epilogue _store :40-49).
+//
+// Shape of the kernel. A workgroup of four wavefronts owns a BM x BN tile of C and walks K in
+// steps of 128 bytes. Per step the A (BM x 128 B) and B (BN x 128 B) slabs live in one of two
+// static LDS stages, filled by direct-to-LDS buffer loads (no staging registers): the loads of
+// step k+1 are issued at the top of step k into the other stage and waited for just before
+// the last MFMA group of step k, where the one barrier of the step sits; the fragments of
+// step k+1 are then read during that last group, so the MFMA pipe has work across the step
+// boundary. Each wavefront computes a (BM/2) x (BN/2) sub-tile as 16x16 MFMA tiles. The
+// MFMA's "A" operand (rows of the 16x16 result) is fed from B (output columns n) and its "B"
+// operand from A (tokens m), so a lane ends up with 4 consecutive n of one m and stores 8
+// bytes of bf16. Rows past M / N are fetched through buffer descriptors whose range check
+// returns zeros.
+//
+// Operand layout of the 16x16x128 MFMA (measured on gfx950 with one-hot operands): lane l
+// carries, for row l%16 and g = l/16, the 16 K bytes [16g, 16g+16) in its first four
+// registers and [64+16g, 64+16g+16) in its last four; the E8M0 byte of lane l scales K block
+// g (bytes [32g, 32g+32)) of row l%16, whichever lanes hold those bytes. The four block
+// scales of a row for one K step are one aligned dword of the natural [rows, K/32] matrix; a
+// lane shifts it right by 8*(l/16) so that byte 0 is the scale it must supply. The faster
+// path reads the MFMA-packed copy (km_scale_pack_offset): for every K step and group of 128
+// rows, 512 bytes ordered [row%16][block][tile=row%128/16], so lane l finds the scale bytes
+// of all eight 16-row tiles of its wave in 8 consecutive bytes at 32*(l%16) + 8*(l/16) and
+// a wavefront fetches them with one coalesced 512-byte load; op_sel then picks the tile.
+//
+// LDS layout of a slab: rows of 128 B = 8 chunks of 16 B. Rows r and r+8 of each group of 16
+// share one 256-byte line (low / high half) and chunk c of row r sits in slot c ^ (r & 7), so
+// the fragment reads (16 lanes = 16 rows at one chunk) touch every bank once. A direct-to-LDS
+// load writes lane i of a wavefront at base + 16*i, so the swizzle is applied on the global
+// side: lane i fetches the chunk whose slot is i & 7.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include <type_traits>
+#include <utility>
+
+#include "km_internal.h"
+#include "km_numeric.h"
+
+namespace km {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kStepBytes = 128;  // K bytes per step (= K elements, e4m3)
+
+__device__ __forceinline__ int slab_offset(int row, int chunk) {
+  return (((row >> 4) * 8 + (row & 7)) << 8) + (((row >> 3) & 1) << 7) + ((chunk ^ (row & 7)) << 4);
+}
+
+template <int OUT>
+__device__ __forceinline__ uint32_t pack2(float a, float b);
+template <>
+__device__ __forceinline__ uint32_t pack2<KM_BF16>(float a, float b) {
+  return f32_to_bf16_bits(a) | (f32_to_bf16_bits(b) << 16);
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<KM_F16>(float a, float b) {
+  _Float16 x = (_Float16)a, y = (_Float16)b;
+  return (uint32_t)__builtin_bit_cast(uint16_t, x) | ((uint32_t)__builtin_bit_cast(uint16_t, y) << 16);
+}
+template <int OUT>
+__device__ __forceinline__ float unpack1(uint32_t h);
+template <>
+__device__ __forceinline__ float unpack1<KM_BF16>(uint32_t h) { return bits_f32(h << 16); }
+template <>
+__device__ __forceinline__ float unpack1<KM_F16>(uint32_t h) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+
+// Work-group id -> (tile_m, tile_n). Work-groups are dealt round-robin to the 8 XCDs, each
+// with its own L2; first give every XCD a contiguous run of tiles, then walk that run in
+// bands of kGroupM row-tiles so that neighbours in time share A rows and B rows in L2.
+constexpr int kXcds = 8;
+constexpr int kGroupM = 8;
+__device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  const int xcd = pid % kXcds, local = pid / kXcds;
+  const int tall = total / kXcds, rem = total % kXcds;
+  int p = xcd < rem ? xcd * (tall + 1) + local : rem * (tall + 1) + (xcd - rem) * tall + local;
+  const int per_group = kGroupM * tiles_n;
+  const int first_m = (p / per_group) * kGroupM;
+  const int group_m = min(tiles_m - first_m, kGroupM);
+  const int in_group = p % per_group;
+  tm = first_m + in_group % group_m;
+  tn = in_group / group_m;
+}
+
+// compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
+
+// c += A(16x128) * B(128x16) with block scales, accumulating in place: the accumulator is an
+// AGPR tuple tied as input and output ("+a"), which keeps all 64 tiles of a wavefront resident
+// in the 256 AGPRs with no copies. op_sel picks which byte of each scale register is used
+// (tile index % 4); it is an immediate, hence one statement per combination.
+#define KM_MFMA_ASM(OSA, OSB, OHA, OHB)                                                              \
+  asm("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[" #OSA "," #OSB ",0] op_sel_hi:[" #OHA "," #OHB ",0]" \
+      : "+a"(c)                                                                                       \
+      : "v"(a), "v"(b), "v"(sa), "v"(sb))
+template <int SEL_A, int SEL_B>
+__device__ __forceinline__ void mfma_acc(v4f& c, const v8i& a, const v8i& b, int sa, int sb) {
+  constexpr int code = (SEL_A & 3) * 4 + (SEL_B & 3);
+  if constexpr (code == 0) KM_MFMA_ASM(0, 0, 0, 0);
+  else if constexpr (code == 1) KM_MFMA_ASM(0, 1, 0, 0);
+  else if constexpr (code == 2) KM_MFMA_ASM(0, 0, 0, 1);
+  else if constexpr (code == 3) KM_MFMA_ASM(0, 1, 0, 1);
+  else if constexpr (code == 4) KM_MFMA_ASM(1, 0, 0, 0);
+  else if constexpr (code == 5) KM_MFMA_ASM(1, 1, 0, 0);
+  else if constexpr (code == 6) KM_MFMA_ASM(1, 0, 0, 1);
+  else if constexpr (code == 7) KM_MFMA_ASM(1, 1, 0, 1);
+  else if constexpr (code == 8) KM_MFMA_ASM(0, 0, 1, 0);
+  else if constexpr (code == 9) KM_MFMA_ASM(0, 1, 1, 0);
+  else if constexpr (code == 10) KM_MFMA_ASM(0, 0, 1, 1);
+  else if constexpr (code == 11) KM_MFMA_ASM(0, 1, 1, 1);
+  else if constexpr (code == 12) KM_MFMA_ASM(1, 0, 1, 0);
+  else if constexpr (code == 13) KM_MFMA_ASM(1, 1, 1, 0);
+  else if constexpr (code == 14) KM_MFMA_ASM(1, 0, 1, 1);
+  else KM_MFMA_ASM(1, 1, 1, 1);
+}
+#undef KM_MFMA_ASM
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// s_waitcnt immediates (gfx9 encoding: vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8])
+constexpr int kWaitVm0 = 0x0F70;         // vmcnt(0)
+constexpr int kWaitVm0Lgkm0 = 0x0070;    // vmcnt(0) lgkmcnt(0)
+
+template <int BM, int BN, bool MX, bool SCALE_KM, int OUT>
+__global__ __launch_bounds__(256) void gemm_fp8_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ As, const uint8_t* __restrict__ B,
+    const uint8_t* __restrict__ Bs, const float* __restrict__ sa, const float* __restrict__ sb,
+    const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N, int K) {
+  constexpr int NT = 256;
+  constexpr int WTM = BM / 2, WTN = BN / 2;
+  constexpr int TM = WTM / 16, TN = WTN / 16;
+  constexpr int A_BYTES = BM * kStepBytes, B_BYTES = BN * kStepBytes;
+  constexpr int STAGE = A_BYTES + B_BYTES;
+  constexpr int A_LD = BM / 32, B_LD = BN / 32;  // 32 rows (4 KiB) per pass of 256 lanes
+  static_assert(BM % 32 == 0 && BN % 32 == 0 && TM >= 1 && TN >= 2, "tile");
+  __shared__ __attribute__((aligned(1024))) uint8_t stage0[STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t stage1[STAGE];
+
+  int tile_m, tile_n;
+  tile_of(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = (wave >> 1) * WTM, wn = (wave & 1) * WTN;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int nk = K / kStepBytes;
+  const int kb = K >> 5;  // scale bytes per row (natural layout)
+
+  // buffer descriptors start at this tile's first row; their range check (on the per-lane
+  // offset) turns rows past the end into zeros
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(A) + (size_t)m0 * K, 0, (int)min((int64_t)(M - m0) * K, (int64_t)0x7FFFFFFF), 0x00020000);
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(B) + (size_t)n0 * K, 0, (int)min((int64_t)(N - n0) * K, (int64_t)0x7FFFFFFF), 0x00020000);
+  // staging map of a pass: 8 lanes per row; 16 lanes cover rows r and r+8 (one LDS line)
+  const int w = tid >> 3;
+  const int srow = ((w >> 4) << 4) + ((w & 1) << 3) + ((w >> 1) & 7);  // 0 .. 31
+  const int src_chunk = (tid & 7) ^ (srow & 7);
+  const int ld_voff = srow * K + src_chunk * 16;
+  const int pass_stride = 32 * K;
+
+  // scales: MFMA rows come from B (n), MFMA columns from A (m)
+  __amdgpu_buffer_rsrc_t ws_rsrc, xs_rsrc;
+  int ws_off[SCALE_KM ? 1 : TN], xs_off[SCALE_KM ? 1 : TM];
+  int ws_step = 0, xs_step = 0, ws_base = 0, xs_base = 0, ws_sel = 0, xs_sel = 0;
+  if constexpr (MX) {
+    if constexpr (SCALE_KM) {
+      // packed: byte offset ((ks*RB + r/128)*16 + r%16)*32 + 8*block + (r%128)/16
+      const int rbn = (N + 127) >> 7, rbm = (M + 127) >> 7;
+      ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(Bs), 0, (int)min((int64_t)nk * rbn * 512, (int64_t)0x7FFFFFFF), 0x00020000);
+      xs_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(As), 0, (int)min((int64_t)nk * rbm * 512, (int64_t)0x7FFFFFFF), 0x00020000);
+      ws_off[0] = r16 * 32 + g * 8;
+      xs_off[0] = ws_off[0];
+      ws_base = min((n0 + wn) >> 7, rbn - 1) * 512;  // waves wholly past the edge read valid bytes
+      xs_base = min((m0 + wm) >> 7, rbm - 1) * 512;
+      ws_step = rbn * 512;
+      xs_step = rbm * 512;
+      ws_sel = (((n0 + wn) & 127) >> 4) * 8;  // bit shift to this wave's first tile
+      xs_sel = (((m0 + wm) & 127) >> 4) * 8;
+    } else {
+      // natural [rows, K/32]; row indices are clamped to the last valid row
+      ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(Bs) + (size_t)n0 * kb, 0,
+                                                  (int)min((int64_t)(N - n0) * kb, (int64_t)0x7FFFFFFF), 0x00020000);
+      xs_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(As) + (size_t)m0 * kb, 0,
+                                                  (int)min((int64_t)(M - m0) * kb, (int64_t)0x7FFFFFFF), 0x00020000);
+      ws_step = 4;
+      xs_step = 4;
+#pragma unroll
+      for (int t = 0; t < TN; ++t) ws_off[t] = min(wn + t * 16 + r16, N - 1 - n0) * kb;
+#pragma unroll
+      for (int t = 0; t < TM; ++t) xs_off[t] = min(wm + t * 16 + r16, M - 1 - m0) * kb;
+    }
+  }
+
+  v4f acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  v8i xf[TM];
+  v8i wcur;
+  // Scale operands of the step being multiplied / raw words of the next step in flight.
+  // Packed layout: two registers per operand hold the bytes of tiles 0-3 and 4-7 (op_sel picks
+  // one); natural layout: one register per tile, its byte 0 is the scale.
+  constexpr int WS = SCALE_KM ? 2 : TN, XS = SCALE_KM ? 2 : TM;
+  // Two sets, one per step parity: a step reads its own set while the next step's set is
+  // written, so no scale register is overwritten while an MFMA that reads it is in flight
+  // (the inline-asm MFMAs are opaque to the compiler's hazard handling).
+  int wscale[2][WS], xscale[2][XS];
+  uint32_t wraw[WS], xraw[XS];
+
+  auto dma = [&](uint8_t* stage, int ks) __attribute__((always_inline)) {
+    const int koff = __builtin_amdgcn_readfirstlane(ks * kStepBytes);
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(stage + i * 4096 + wave * 1024), 16,
+                                               ld_voff + i * pass_stride, koff, 0, 0);
+#pragma unroll
+    for (int i = 0; i < B_LD; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(stage + A_BYTES + i * 4096 + wave * 1024), 16,
+                                               ld_voff + i * pass_stride, koff, 0, 0);
+  };
+  auto scale_fetch = [&](int ks) __attribute__((always_inline)) {
+    if constexpr (MX) {
+      const int wso = __builtin_amdgcn_readfirstlane(ks * ws_step + ws_base);
+      const int xso = __builtin_amdgcn_readfirstlane(ks * xs_step + xs_base);
+      if constexpr (SCALE_KM) {
+        const uint2 wv = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(ws_rsrc, ws_off[0], wso, 0));
+        const uint2 xv = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(xs_rsrc, xs_off[0], xso, 0));
+        wraw[0] = wv.x; wraw[1] = wv.y;
+        xraw[0] = xv.x; xraw[1] = xv.y;
+      } else {
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+          wraw[t] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ws_rsrc, ws_off[t], wso, 0);
+#pragma unroll
+        for (int t = 0; t < TM; ++t)
+          xraw[t] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(xs_rsrc, xs_off[t], xso, 0);
+      }
+    }
+  };
+  // `live` is all ones for a real step and zero for the padding step of an odd step count:
+  // zero scale bytes (2^-127 on both sides) make that step add exactly 0.
+  auto scale_commit = [&](auto set_tag, uint32_t live) __attribute__((always_inline)) {
+    constexpr int P = decltype(set_tag)::value;
+    if constexpr (!MX) {
+#pragma unroll
+      for (int t = 0; t < WS; ++t) wscale[P][t] = (int)(0x7F7F7F7Fu & live);
+#pragma unroll
+      for (int t = 0; t < XS; ++t) xscale[P][t] = (int)(0x7F7F7F7Fu & live);
+    } else if constexpr (SCALE_KM) {
+      const uint64_t wv = (((uint64_t)wraw[1] << 32) | wraw[0]) >> ws_sel;
+      const uint64_t xv = (((uint64_t)xraw[1] << 32) | xraw[0]) >> xs_sel;
+      wscale[P][0] = (int)((uint32_t)wv & live); wscale[P][1] = (int)((uint32_t)(wv >> 32) & live);
+      xscale[P][0] = (int)((uint32_t)xv & live); xscale[P][1] = (int)((uint32_t)(xv >> 32) & live);
+    } else {
+#pragma unroll
+      for (int t = 0; t < TN; ++t) wscale[P][t] = (int)((wraw[t] >> (8 * g)) & live);
+#pragma unroll
+      for (int t = 0; t < TM; ++t) xscale[P][t] = (int)((xraw[t] >> (8 * g)) & live);
+    }
+  };
+  auto fragment = [&](const uint8_t* slab, int row) __attribute__((always_inline)) -> v8i {
+    const v4i lo = *reinterpret_cast<const v4i*>(slab + slab_offset(row, g));
+    const v4i hi = *reinterpret_cast<const v4i*>(slab + slab_offset(row, g + 4));
+    return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
+  // One K step out of `cur` with scale set P. Step ks+1 (clamped to the last one) is fetched
+  // into `nxt` meanwhile; its first fragments are read after the barrier, during the last MFMA
+  // group (each fragment register is reloaded one MFMA after the last MFMA that read it), and
+  // its scales are committed to set P^1.
+  auto step = [&](uint8_t* cur, uint8_t* nxt, int ks, auto set_tag) __attribute__((always_inline)) {
+    constexpr int P = decltype(set_tag)::value;
+    const int next = min(ks + 1, nk - 1);
+    dma(nxt, next);
+    scale_fetch(next);
+    __builtin_amdgcn_sched_barrier(0);  // keep the fetches at the top of the step
+    static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
+      constexpr int t = decltype(t_tag)::value;
+      v8i wnext;
+      if constexpr (t + 1 < TN) {
+        wnext = fragment(cur + A_BYTES, wn + (t + 1) * 16 + r16);
+      } else {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        wnext = fragment(nxt + A_BYTES, wn + r16);
+      }
+      static_for<TM>([&](auto j_tag) __attribute__((always_inline)) {
+        constexpr int j = decltype(j_tag)::value;
+        if constexpr (SCALE_KM)
+          mfma_acc<t, j>(acc[t][j], wcur, xf[j], wscale[P][(t >> 2) % WS], xscale[P][(j >> 2) % XS]);
+        else
+          mfma_acc<0, 0>(acc[t][j], wcur, xf[j], wscale[P][t % WS], xscale[P][j % XS]);
+        if constexpr (t + 1 == TN && j >= 1) {
+          __builtin_amdgcn_sched_barrier(0);
+          xf[j - 1] = fragment(nxt, wm + (j - 1) * 16 + r16);
+        }
+      });
+      if constexpr (t + 1 == TN) {
+        __builtin_amdgcn_sched_barrier(0);
+        xf[TM - 1] = fragment(nxt, wm + (TM - 1) * 16 + r16);
+      }
+      wcur = wnext;
+    });
+    scale_commit(std::integral_constant<int, P ^ 1>{}, ks + 1 < nk ? 0xFFFFFFFFu : 0u);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using set0_t = std::integral_constant<int, 0>;
+  using set1_t = std::integral_constant<int, 1>;
+
+  // prologue: step 0 into stage0, scale set 0
+  dma(stage0, 0);
+  scale_fetch(0);
+  __builtin_amdgcn_s_waitcnt(kWaitVm0);
+  __syncthreads();
+  scale_commit(set0_t{}, 0xFFFFFFFFu);
+#pragma unroll
+  for (int j = 0; j < TM; ++j) xf[j] = fragment(stage0, wm + j * 16 + r16);
+  wcur = fragment(stage0 + A_BYTES, wn + r16);
+
+  // two steps per trip, one per stage; an odd step count is padded with a zero-scaled step
+  const int nsteps = (nk + 1) & ~1;
+  for (int ks = 0; ks < nsteps; ks += 2) {
+    step(stage0, stage1, ks, set0_t{});
+    step(stage1, stage0, ks + 1, set1_t{});
+  }
+
+  // the MFMAs above are opaque to the compiler's hazard handling: give the last ones time to
+  // retire before the accumulators are read
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+
+  // epilogue: lane holds C[m][n .. n+3] for m = m0+wm+j*16+r16, n = n0+wn+t*16+4*g
+  float post = 1.0f;
+  if constexpr (!MX) post = sa[0] * sb[0];
+  const bool vec_ok = (N & 3) == 0;
+#pragma unroll
+  for (int t = 0; t < TN; ++t) {
+    const int n = n0 + wn + t * 16 + 4 * g;
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias != nullptr) {
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        if (n + v < N) bv[v] = unpack1<OUT>(bias[n + v]);
+    }
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      const int m = m0 + wm + j * 16 + r16;
+      if (m >= M || n >= N) continue;
+      float o[4];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) o[v] = MX ? acc[t][j][v] + bv[v] : acc[t][j][v] * post + bv[v];
+      uint16_t* dst = C + (size_t)m * N + n;
+      if (vec_ok && n + 3 < N) {
+        *reinterpret_cast<uint2*>(dst) = make_uint2(pack2<OUT>(o[0], o[1]), pack2<OUT>(o[2], o[3]));
+      } else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (n + v < N) dst[v] = (uint16_t)(pack2<OUT>(o[v], 0.f) & 0xFFFFu);
+      }
+    }
+  }
+}
+
+struct GemmConfig {
+  int bm, bn;
+};
+// Largest tile first: the host-side table ranks candidates the way the reference ranks its
+// Triton tiles (large tiles for large M). Four wavefronts in a 2 x 2 grid each.
+static const GemmConfig kGemmConfigs[] = {
+    {256, 256},
+    {128, 256},
+    {256, 128},
+    {128, 128},
+    {64, 128},
+};
+constexpr int kNumGemmConfigs = sizeof(kGemmConfigs) / sizeof(kGemmConfigs[0]);
+
+template <int BM, int BN, bool MX, bool SCALE_KM, int OUT>
+static int launch_gemm(const void* a, const void* as, const void* b, const void* bs, const float* sa,
+                       const float* sb, const void* bias, void* c, int M, int N, int K,
+                       hipStream_t st) {
+  const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  hipLaunchKernelGGL((gemm_fp8_kernel<BM, BN, MX, SCALE_KM, OUT>), dim3(tiles), dim3(256), 0, st,
+                     (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b, (const uint8_t*)bs, sa, sb,
+                     (const uint16_t*)bias, (uint16_t*)c, M, N, K);
+  return km_check_launch("km_gemm");
+}
+
+template <bool MX, bool SCALE_KM, int OUT>
+static int dispatch_config(int config, const void* a, const void* as, const void* b, const void* bs,
+                           const float* sa, const float* sb, const void* bias, void* c, int M, int N,
+                           int K, hipStream_t st) {
+  switch (config) {
+    case 0: return launch_gemm<256, 256, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
+    case 1: return launch_gemm<128, 256, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
+    case 2: return launch_gemm<256, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
+    case 3: return launch_gemm<128, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
+    case 4: return launch_gemm<64, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
+  }
+  return km_fail(KM_ERR_ARG, "km_gemm: unknown config");
+}
+
+static int check_gemm_args(const char* who, const void* a, const void* b, void* c, int64_t M, int64_t N,
+                           int64_t K, int out_dtype, int config) {
+  static thread_local char msg[160];
+  if (out_dtype != KM_BF16 && out_dtype != KM_F16) {
+    snprintf(msg, sizeof msg, "%s: out_dtype must be bf16 or f16", who);
+    return km_fail(KM_ERR_ARG, msg);
+  }
+  if (M < 0 || N < 0 || K <= 0 || K % kStepBytes) {
+    snprintf(msg, sizeof msg, "%s: K=%lld must be a positive multiple of 128", who, (long long)K);
+    return km_fail(KM_ERR_UNSUPPORTED, msg);
+  }
+  if (M * K > 0x7FFFFFFFll || N * K > 0x7FFFFFFFll || M > 0x0FFFFFFF || N > 0x0FFFFFFF) {
+    snprintf(msg, sizeof msg, "%s: dimension too large", who);
+    return km_fail(KM_ERR_ARG, msg);
+  }
+  if (config < 0 || config >= kNumGemmConfigs) {
+    snprintf(msg, sizeof msg, "%s: config %d out of range", who, config);
+    return km_fail(KM_ERR_ARG, msg);
+  }
+  if (M > 0 && N > 0 && (!a || !b || !c)) {
+    snprintf(msg, sizeof msg, "%s: null pointer", who);
+    return km_fail(KM_ERR_ARG, msg);
+  }
+  if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) {
+    snprintf(msg, sizeof msg, "%s: operands must be 16-byte aligned", who);
+    return km_fail(KM_ERR_UNSUPPORTED, msg);
+  }
+  return KM_OK;
+}
+
+int gemm_num_configs() { return kNumGemmConfigs; }
+int gemm_config_desc(int config, char* buf, int len) {
+  if (config < 0 || config >= kNumGemmConfigs) return km_fail(KM_ERR_ARG, "config out of range");
+  const GemmConfig& c = kGemmConfigs[config];
+  snprintf(buf, len, "bm=%d,bn=%d,bk=128,waves=4", c.bm, c.bn);
+  return KM_OK;
+}
+
+}  // namespace km
+
+using namespace km;
+
+extern "C" int km_gemm_mx(const void* a, const void* a_scale, const void* b, const void* b_scale,
+                          const void* bias, void* c, int64_t M, int64_t N, int64_t K, int out_dtype,
+                          int scale_layout, int config, void* stream) {
+  int rc = check_gemm_args("km_gemm_mx", a, b, c, M, N, K, out_dtype, config);
+  if (rc != KM_OK) return rc;
+  if (M == 0 || N == 0) return KM_OK;
+  if (!a_scale || !b_scale) return km_fail(KM_ERR_ARG, "km_gemm_mx: null scale pointer");
+  if (scale_layout != KM_SCALES_ROWMAJOR && scale_layout != KM_SCALES_PACKED)
+    return km_fail(KM_ERR_ARG, "km_gemm_mx: unknown scale layout");
+  if ((reinterpret_cast<uintptr_t>(a_scale) | reinterpret_cast<uintptr_t>(b_scale)) & 3)
+    return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_mx: scales must be 4-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  const bool km = scale_layout == KM_SCALES_PACKED;
+  if (out_dtype == KM_BF16) {
+    if (km) return dispatch_config<true, true, KM_BF16>(config, a, a_scale, b, b_scale, nullptr, nullptr, bias, c, (int)M, (int)N, (int)K, st);
+    return dispatch_config<true, false, KM_BF16>(config, a, a_scale, b, b_scale, nullptr, nullptr, bias, c, (int)M, (int)N, (int)K, st);
+  }
+  if (km) return dispatch_config<true, true, KM_F16>(config, a, a_scale, b, b_scale, nullptr, nullptr, bias, c, (int)M, (int)N, (int)K, st);
+  return dispatch_config<true, false, KM_F16>(config, a, a_scale, b, b_scale, nullptr, nullptr, bias, c, (int)M, (int)N, (int)K, st);
+}
+
+extern "C" int km_gemm_fp8_tensor(const void* a, const float* sa, const void* b, const float* sb,
+                                  const void* bias, void* c, int64_t M, int64_t N, int64_t K,
+                                  int out_dtype, int config, void* stream) {
+  int rc = check_gemm_args("km_gemm_fp8_tensor", a, b, c, M, N, K, out_dtype, config);
+  if (rc != KM_OK) return rc;
+  if (M == 0 || N == 0) return KM_OK;
+  if (!sa || !sb) return km_fail(KM_ERR_ARG, "km_gemm_fp8_tensor: null scale pointer");
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == KM_BF16)
+    return dispatch_config<false, false, KM_BF16>(config, a, nullptr, b, nullptr, sa, sb, bias, c, (int)M, (int)N, (int)K, st);
+  return dispatch_config<false, false, KM_F16>(config, a, nullptr, b, nullptr, sa, sb, bias, c, (int)M, (int)N, (int)K, st);
+}

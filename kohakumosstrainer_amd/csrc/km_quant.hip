@@ -1,0 +1,427 @@
+// Activation / weight quantizers for gfx950: bandwidth kernels.
+//
+//   quant_mx_rows     MXFP8 along a unit-stride contraction axis (reference
+//                     src/kohakumoss_kernels/fp8/formats.py:94-99; the Triton kernel it
+//                     replaces is backends/triton/fp8/quantize.py:94-118)
+//   quant_mx_cols     MXFP8 of the transposed view (blocks run along the strided axis of
+//                     the input), what `quantize(x.t(), "mx")` computes for the input-
+//                     gradient weight copy (reference src/kohakumoss/quant/compute.py:63-66)
+//   quant_mx_generic  any strides, one thread per block of 32
+//   tensor_amax / tensor_cast   per-tensor recipe (reference formats.py:77-79,
+//                     Triton quantize.py:86-91,161-168)
+//
+// All of them read each input element once and write each output byte once.
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "km_internal.h"
+#include "km_numeric.h"
+
+namespace km {
+
+template <int DT>
+__device__ __forceinline__ float widen(uint32_t h);
+template <>
+__device__ __forceinline__ float widen<KM_BF16>(uint32_t h) { return bits_f32(h << 16); }
+template <>
+__device__ __forceinline__ float widen<KM_F16>(uint32_t h) {
+  return __half2float(__ushort_as_half((unsigned short)h));
+}
+
+// Byte offset of scale (row, block) in the MFMA-packed layout the GEMM reads: per K step of
+// 128 and group of 128 rows, 512 bytes ordered [row%16][block%4][row%128/16].
+__device__ __forceinline__ uint64_t scale_pack_offset(uint64_t row, uint64_t block, uint64_t row_groups) {
+  return ((((block >> 2) * row_groups + (row >> 7)) * 16 + (row & 15)) * 4 + (block & 3)) * 8 + ((row & 127) >> 4);
+}
+
+// max over the 4 lanes of a quad, every lane of the quad gets it (DPP quad_perm swaps).
+__device__ __forceinline__ uint32_t quad_max(uint32_t v) {
+  uint32_t o = (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);  // [1,0,3,2]
+  v = v > o ? v : o;
+  o = (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xF, 0xF, true);  // [2,3,0,1]
+  return v > o ? v : o;
+}
+
+// 8 values (one 128-bit load) -> 8 fp32
+template <int DT>
+__device__ __forceinline__ void widen8(const uint4& raw, float (&f)[8]) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = widen<DT>(w[i] & 0xFFFFu);
+    f[2 * i + 1] = widen<DT>(w[i] >> 16);
+  }
+}
+
+__device__ __forceinline__ uint32_t amax_bits8(const float (&f)[8]) {
+  uint32_t m = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    uint32_t a = f32_bits(f[i]) & kAbsMask;
+    m = a > m ? a : m;
+  }
+  return m;
+}
+
+__device__ __forceinline__ uint2 encode8(const float (&f)[8], float inv) {
+  uint32_t lo = 0, hi = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    lo |= e4m3_encode(f[i] * inv) << (8 * i);
+    hi |= e4m3_encode(f[4 + i] * inv) << (8 * i);
+  }
+  return make_uint2(lo, hi);
+}
+
+// ---- rows: lane = 8 consecutive elements, quad = one block of 32 --------------------------
+// Group g (8 elements) of row g / groups_per_row; outputs are flat because q and the
+// scales are contiguous row-major. UNROLL independent 128-bit loads are in flight per lane.
+constexpr int kRowsThreads = 256;
+constexpr int kRowsUnroll = 4;
+
+// byte of lane i+4, i+8, i+12 of the same 16-lane row gathered into one dword (lane i%16 == 0
+// ends up with the four scale bytes of four consecutive blocks)
+__device__ __forceinline__ uint32_t gather4_stride4(uint32_t b) {
+  uint32_t v = b & 0xFFu;
+  v |= ((uint32_t)__builtin_amdgcn_mov_dpp((int)b, 0x104, 0xF, 0xF, true) & 0xFFu) << 8;   // row_shl:4
+  v |= ((uint32_t)__builtin_amdgcn_mov_dpp((int)b, 0x108, 0xF, 0xF, true) & 0xFFu) << 16;  // row_shl:8
+  v |= ((uint32_t)__builtin_amdgcn_mov_dpp((int)b, 0x10C, 0xF, 0xF, true) & 0xFFu) << 24;  // row_shl:12
+  return v;
+}
+
+// PACK4: cols % 128 == 0, so the 16 lanes of a DPP row cover four consecutive blocks of one
+// row and their natural-layout scale bytes are stored as one dword.
+template <int DT, bool PACK4>
+__global__ __launch_bounds__(kRowsThreads) void quant_mx_rows(
+    const uint16_t* __restrict__ x, int64_t ld, uint32_t groups_per_row, uint64_t ngroups, uint32_t rows,
+    uint8_t* __restrict__ q, uint8_t* __restrict__ scales, uint8_t* __restrict__ scales_km) {
+  const uint64_t base = (uint64_t)blockIdx.x * (kRowsThreads * kRowsUnroll) + threadIdx.x;
+  const bool dense = ld == (int64_t)groups_per_row * 8;
+  uint4 raw[kRowsUnroll];
+#pragma unroll
+  for (int u = 0; u < kRowsUnroll; ++u) {
+    const uint64_t g = base + (uint64_t)u * kRowsThreads;
+    raw[u] = make_uint4(0, 0, 0, 0);
+    if (g < ngroups) {
+      uint64_t off;
+      if (dense) {
+        off = g * 8;
+      } else {
+        const uint64_t row = g / groups_per_row;
+        off = row * (uint64_t)ld + (g - row * groups_per_row) * 8;
+      }
+      raw[u] = *reinterpret_cast<const uint4*>(x + off);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kRowsUnroll; ++u) {
+    const uint64_t g = base + (uint64_t)u * kRowsThreads;
+    float f[8];
+    widen8<DT>(raw[u], f);
+    const uint32_t biased = mx_biased_exponent(quad_max(amax_bits8(f)));
+    const uint2 codes = encode8(f, mx_inverse_scale(biased));
+    if constexpr (PACK4) {
+      const uint32_t four = gather4_stride4(biased);
+      if (g < ngroups) {
+        *reinterpret_cast<uint2*>(q + g * 8) = codes;
+        if (scales && (threadIdx.x & 15) == 0) reinterpret_cast<uint32_t*>(scales)[g >> 4] = four;
+        if (scales_km && (threadIdx.x & 3) == 0) {
+          const uint32_t blocks = groups_per_row >> 2;
+          const uint64_t b = g >> 2;
+          const uint64_t row = b / blocks;
+          scales_km[scale_pack_offset(row, b - row * blocks, (rows + 127) >> 7)] = (uint8_t)biased;
+        }
+      }
+    } else {
+      if (g < ngroups) {
+        *reinterpret_cast<uint2*>(q + g * 8) = codes;
+        if ((threadIdx.x & 3) == 0) scales[g >> 2] = (uint8_t)biased;
+      }
+    }
+  }
+}
+
+// ---- cols: blocks run along the strided axis ------------------------------------------------
+// Input x[r][c] (c unit stride); output q_t[c][r], scales_t[c][r/32]. A workgroup stages a
+// TR x TC tile in LDS with 128-bit row loads, then each lane owns two adjacent columns of one
+// 32-row block: it reads 32 dwords down the tile, reduces in registers and writes two
+// 32-byte runs of q_t.
+constexpr int kColsThreads = 256;
+constexpr int kColsTR = 256;  // rows of x per tile (8 blocks)
+constexpr int kColsTC = 64;   // columns of x per tile
+constexpr int kColsPitch = kColsTC / 2 + 4;  // dwords per staged row (16-byte aligned rows)
+constexpr int kColsSkew = 8;  // extra dwords after each 32 rows: spreads the 8 blocks over banks
+
+template <int DT>
+__global__ __launch_bounds__(kColsThreads) void quant_mx_cols(
+    const uint16_t* __restrict__ x, int64_t ld, int64_t rows, int64_t cols,
+    uint8_t* __restrict__ q_t, uint8_t* __restrict__ scales_t, uint8_t* __restrict__ scales_km) {
+  __shared__ __attribute__((aligned(16))) uint32_t tile[kColsTR * kColsPitch + (kColsTR / 32) * kColsSkew];
+  const int64_t r0 = (int64_t)blockIdx.y * kColsTR;
+  const int64_t c0 = (int64_t)blockIdx.x * kColsTC;
+  const int tid = threadIdx.x;
+  // stage: 8 lanes cover one 128-byte row segment
+  {
+    const int cg = tid & 7;   // 8-element group within the row segment
+    const int rr = tid >> 3;  // 0..31
+    uint4 raw[kColsTR / 32];
+#pragma unroll
+    for (int i = 0; i < kColsTR / 32; ++i) {
+      const int64_t r = r0 + rr + 32 * i;
+      const int64_t c = c0 + cg * 8;
+      raw[i] = make_uint4(0, 0, 0, 0);
+      if (r < rows && c < cols) raw[i] = *reinterpret_cast<const uint4*>(x + r * ld + c);
+    }
+#pragma unroll
+    for (int i = 0; i < kColsTR / 32; ++i) {
+      const int lr = rr + 32 * i;
+      *reinterpret_cast<uint4*>(&tile[lr * kColsPitch + i * kColsSkew + cg * 4]) = raw[i];
+    }
+  }
+  __syncthreads();
+  // lane -> (block of 32 rows, column pair); blocks vary fastest so a wave writes runs of
+  // consecutive bytes of q_t rows
+  const int blk = tid & 7;
+  const int pair = tid >> 3;  // 0..31
+  const int64_t rb = r0 + blk * 32;
+  const int64_t c = c0 + pair * 2;
+  if (rb >= rows || c >= cols) return;
+  const uint32_t* col = &tile[blk * 32 * kColsPitch + blk * kColsSkew + pair];
+  uint32_t w[32];
+#pragma unroll
+  for (int i = 0; i < 32; ++i) w[i] = col[i * kColsPitch];
+  uint32_t m0 = 0, m1 = 0;
+  float f0[32], f1[32];
+#pragma unroll
+  for (int i = 0; i < 32; ++i) {
+    f0[i] = widen<DT>(w[i] & 0xFFFFu);
+    f1[i] = widen<DT>(w[i] >> 16);
+    const uint32_t a0 = f32_bits(f0[i]) & kAbsMask, a1 = f32_bits(f1[i]) & kAbsMask;
+    m0 = a0 > m0 ? a0 : m0;
+    m1 = a1 > m1 ? a1 : m1;
+  }
+  const uint32_t b0 = mx_biased_exponent(m0), b1 = mx_biased_exponent(m1);
+  const float i0 = mx_inverse_scale(b0), i1 = mx_inverse_scale(b1);
+  uint32_t o0[8], o1[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    o0[j] = o1[j] = 0;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      o0[j] |= e4m3_encode(f0[4 * j + t] * i0) << (8 * t);
+      o1[j] |= e4m3_encode(f1[4 * j + t] * i1) << (8 * t);
+    }
+  }
+  uint4* d0 = reinterpret_cast<uint4*>(q_t + c * rows + rb);
+  d0[0] = make_uint4(o0[0], o0[1], o0[2], o0[3]);
+  d0[1] = make_uint4(o0[4], o0[5], o0[6], o0[7]);
+  // logical operand is [cols][rows]: row index c, block index rb / 32
+  const int64_t nblk = rows / 32;
+  const int64_t lb = rb / 32;
+  if (scales_t) scales_t[c * nblk + lb] = (uint8_t)b0;
+  if (scales_km) scales_km[scale_pack_offset(c, lb, (cols + 127) >> 7)] = (uint8_t)b0;
+  if (c + 1 < cols) {
+    uint4* d1 = reinterpret_cast<uint4*>(q_t + (c + 1) * rows + rb);
+    d1[0] = make_uint4(o1[0], o1[1], o1[2], o1[3]);
+    d1[1] = make_uint4(o1[4], o1[5], o1[6], o1[7]);
+    if (scales_t) scales_t[(c + 1) * nblk + lb] = (uint8_t)b1;
+    if (scales_km) scales_km[scale_pack_offset(c + 1, lb, (cols + 127) >> 7)] = (uint8_t)b1;
+  }
+}
+
+// ---- generic: any strides, one thread per block ----------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(256) void quant_mx_generic(
+    const uint16_t* __restrict__ x, int64_t sr, int64_t sc, int64_t rows, int64_t cols,
+    uint8_t* __restrict__ q, uint8_t* __restrict__ scales, uint8_t* __restrict__ scales_km) {
+  const int64_t nblk = cols / 32;
+  const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (b >= rows * nblk) return;
+  const int64_t r = b / nblk, cb = b - r * nblk;
+  const uint16_t* src = x + r * sr + cb * 32 * sc;
+  float f[32];
+  uint32_t m = 0;
+#pragma unroll
+  for (int i = 0; i < 32; ++i) {
+    f[i] = widen<DT>(src[i * sc]);
+    const uint32_t a = f32_bits(f[i]) & kAbsMask;
+    m = a > m ? a : m;
+  }
+  const uint32_t biased = mx_biased_exponent(m);
+  const float inv = mx_inverse_scale(biased);
+  uint8_t* dst = q + r * cols + cb * 32;
+#pragma unroll
+  for (int i = 0; i < 32; ++i) dst[i] = (uint8_t)e4m3_encode(f[i] * inv);
+  if (scales) scales[b] = (uint8_t)biased;
+  if (scales_km) scales_km[scale_pack_offset(r, cb, (rows + 127) >> 7)] = (uint8_t)biased;
+}
+
+// natural scales [rows, blocks] -> MFMA-packed; one byte per thread
+__global__ __launch_bounds__(256) void scales_pack(const uint8_t* __restrict__ in, int64_t rows, int64_t blocks,
+                                                   uint8_t* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= rows * blocks) return;
+  const int64_t r = i / blocks, b = i - r * blocks;
+  out[scale_pack_offset(r, b, (rows + 127) >> 7)] = in[i];
+}
+
+// ---- per-tensor recipe -----------------------------------------------------------------------
+__global__ void fill_u32(uint32_t* p, uint32_t v) { *p = v; }
+
+template <int DT>
+__global__ __launch_bounds__(256) void tensor_amax(const uint16_t* __restrict__ x, int64_t sr,
+                                                   int64_t sc, int64_t rows, int64_t cols,
+                                                   uint32_t* __restrict__ amax_bits) {
+  // non-negative floats order like their bits: an unsigned atomic max is an abs-max
+  const int64_t n = rows * cols;
+  const bool dense = sc == 1 && sr == cols;
+  uint32_t m = 0;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  if (dense && (cols % 8) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < n / 8; g += stride) {
+      float f[8];
+      widen8<DT>(reinterpret_cast<const uint4*>(x)[g], f);
+      const uint32_t a = amax_bits8(f);
+      m = a > m ? a : m;
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+      const int64_t r = i / cols, c = i - r * cols;
+      const uint32_t a = f32_bits(widen<DT>(x[r * sr + c * sc])) & kAbsMask;
+      m = a > m ? a : m;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const uint32_t o = (uint32_t)__shfl_xor((int)m, off);
+    m = o > m ? o : m;
+  }
+  if ((threadIdx.x & 63) == 0 && m != 0) atomicMax(amax_bits, m);
+}
+
+// s = max(amax, 1e-12) / 448 and q = e4m3(clamp(x / s)), both IEEE fp32 divisions.
+template <int DT>
+__global__ __launch_bounds__(256) void tensor_cast(const uint16_t* __restrict__ x, int64_t sr,
+                                                   int64_t sc, int64_t rows, int64_t cols,
+                                                   const uint32_t* __restrict__ amax_bits,
+                                                   uint8_t* __restrict__ q,
+                                                   float* __restrict__ scale_out) {
+  uint32_t ab = *amax_bits;
+  ab = ab > kAmaxFloorBits ? ab : kAmaxFloorBits;
+  const float s = __fdiv_rn(bits_f32(ab), 448.0f);
+  if (blockIdx.x == 0 && threadIdx.x == 0 && scale_out) *scale_out = s;
+  const int64_t n = rows * cols;
+  const bool dense = sc == 1 && sr == cols;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  if (dense && (cols % 8) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < n / 8; g += stride) {
+      float f[8];
+      widen8<DT>(reinterpret_cast<const uint4*>(x)[g], f);
+      uint32_t lo = 0, hi = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        lo |= e4m3_encode(__fdiv_rn(f[i], s)) << (8 * i);
+        hi |= e4m3_encode(__fdiv_rn(f[4 + i], s)) << (8 * i);
+      }
+      reinterpret_cast<uint2*>(q)[g] = make_uint2(lo, hi);
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+      const int64_t r = i / cols, c = i - r * cols;
+      q[i] = (uint8_t)e4m3_encode(__fdiv_rn(widen<DT>(x[r * sr + c * sc]), s));
+    }
+  }
+}
+
+}  // namespace km
+
+using namespace km;
+
+#define KM_DISPATCH_DT(dt, ...)                       \
+  if ((dt) == KM_BF16) {                              \
+    constexpr int DT = KM_BF16;                       \
+    __VA_ARGS__;                                      \
+  } else {                                            \
+    constexpr int DT = KM_F16;                        \
+    __VA_ARGS__;                                      \
+  }
+
+extern "C" int km_quant_mx(const void* x, int64_t rows, int64_t cols, int64_t stride_row,
+                           int64_t stride_col, int dtype, void* q, void* scales, void* scales_packed,
+                           void* stream) {
+  if (dtype != KM_BF16 && dtype != KM_F16) return km_fail(KM_ERR_ARG, "km_quant_mx: dtype must be bf16 or f16");
+  if (rows < 0 || cols < 0 || cols % 32) return km_fail(KM_ERR_ARG, "km_quant_mx: cols must be a non-negative multiple of 32");
+  if (scales_packed && cols % 128) return km_fail(KM_ERR_ARG, "km_quant_mx: the packed scale copy needs cols % 128 == 0");
+  if (rows == 0 || cols == 0) return KM_OK;
+  if (!x || !q || (!scales && !scales_packed)) return km_fail(KM_ERR_ARG, "km_quant_mx: null pointer");
+  if (reinterpret_cast<uintptr_t>(scales) & 3) return km_fail(KM_ERR_ARG, "km_quant_mx: scales must be 4-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  const uint16_t* xp = (const uint16_t*)x;
+  uint8_t *qp = (uint8_t*)q, *sp = (uint8_t*)scales, *kp = (uint8_t*)scales_packed;
+  const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 15) == 0;
+  const uint64_t ngroups = (uint64_t)rows * (uint64_t)cols / 8;
+  if (stride_col == 1 && aligned && stride_row % 8 == 0 && stride_row >= cols && ngroups < (1ull << 40) && rows < (1ll << 31)) {
+    const uint64_t per_block = (uint64_t)kRowsThreads * kRowsUnroll;
+    const uint64_t blocks = (ngroups + per_block - 1) / per_block;
+    if (blocks > 0x7FFFFFFFull) return km_fail(KM_ERR_ARG, "km_quant_mx: tensor too large");
+    const bool pack4 = cols % 128 == 0;
+    if (!pack4 && !sp) return km_fail(KM_ERR_ARG, "km_quant_mx: null scales");
+    KM_DISPATCH_DT(dtype, {
+      if (pack4)
+        hipLaunchKernelGGL((quant_mx_rows<DT, true>), dim3((unsigned)blocks), dim3(kRowsThreads), 0, st, xp, stride_row,
+                           (uint32_t)(cols / 8), ngroups, (uint32_t)rows, qp, sp, kp);
+      else
+        hipLaunchKernelGGL((quant_mx_rows<DT, false>), dim3((unsigned)blocks), dim3(kRowsThreads), 0, st, xp, stride_row,
+                           (uint32_t)(cols / 8), ngroups, (uint32_t)rows, qp, sp, kp);
+    });
+  } else if (stride_row == 1 && aligned && stride_col % 8 == 0 && stride_col >= rows && rows % 8 == 0) {
+    // the memory is a row-major [cols][rows] matrix read along its unit-stride axis; blocks of
+    // 32 run down its rows
+    const int64_t mem_rows = cols, mem_cols = rows;
+    dim3 grid((unsigned)((mem_cols + kColsTC - 1) / kColsTC), (unsigned)((mem_rows + kColsTR - 1) / kColsTR));
+    if (grid.y > 65535u) return km_fail(KM_ERR_ARG, "km_quant_mx: tensor too large for the transposing kernel");
+    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL(quant_mx_cols<DT>, grid, dim3(kColsThreads), 0, st, xp, stride_col,
+                                             mem_rows, mem_cols, qp, sp, kp));
+  } else {
+    const int64_t nb = rows * (cols / 32);
+    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL(quant_mx_generic<DT>, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, st,
+                                             xp, stride_row, stride_col, rows, cols, qp, sp, kp));
+  }
+  return km_check_launch("km_quant_mx");
+}
+
+extern "C" int64_t km_scales_packed_bytes(int64_t rows, int64_t cols) {
+  if (rows < 0 || cols < 0 || cols % 128) return -1;
+  return (cols / 128) * ((rows + 127) / 128) * 512;
+}
+
+extern "C" int km_scales_pack(const void* scales, int64_t rows, int64_t cols, void* out, void* stream) {
+  if (rows < 0 || cols < 0 || cols % 128) return km_fail(KM_ERR_ARG, "km_scales_pack: cols must be a multiple of 128");
+  if (rows == 0 || cols == 0) return KM_OK;
+  if (!scales || !out) return km_fail(KM_ERR_ARG, "km_scales_pack: null pointer");
+  const int64_t n = rows * (cols / 32);
+  hipLaunchKernelGGL(scales_pack, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const uint8_t*)scales, rows, cols / 32, (uint8_t*)out);
+  return km_check_launch("km_scales_pack");
+}
+
+extern "C" int km_quant_tensor(const void* x, int64_t rows, int64_t cols, int64_t stride_row,
+                               int64_t stride_col, int dtype, void* q, float* scale_out,
+                               uint32_t* amax_workspace, void* stream) {
+  if (dtype != KM_BF16 && dtype != KM_F16) return km_fail(KM_ERR_ARG, "km_quant_tensor: dtype must be bf16 or f16");
+  if (rows < 0 || cols < 0) return km_fail(KM_ERR_ARG, "km_quant_tensor: negative shape");
+  if (!scale_out || !amax_workspace) return km_fail(KM_ERR_ARG, "km_quant_tensor: null scale or workspace");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t n = rows * cols;
+  if (n > 0 && (!x || !q)) return km_fail(KM_ERR_ARG, "km_quant_tensor: null pointer");
+  hipLaunchKernelGGL(fill_u32, dim3(1), dim3(1), 0, st, amax_workspace, 0u);
+  int64_t want = (n / 8 + 255) / 256;
+  unsigned blocks = (unsigned)(want < 1 ? 1 : (want > 8192 ? 8192 : want));
+  const uint16_t* xp = (const uint16_t*)x;
+  KM_DISPATCH_DT(dtype, {
+    if (n > 0) hipLaunchKernelGGL(tensor_amax<DT>, dim3(blocks), dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, amax_workspace);
+    hipLaunchKernelGGL(tensor_cast<DT>, dim3(blocks), dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, amax_workspace, (uint8_t*)q, scale_out);
+  });
+  return km_check_launch("km_quant_tensor");
+}

@@ -1,0 +1,318 @@
+"""ctypes binding of libkm_kernels.so (hand-written HIP for gfx950) and thin tensor-level
+wrappers. torch is used for device memory and the current stream only.
+
+Every wrapper validates shapes / dtypes / devices on the host before a launch, allocates
+its outputs, launches on torch's current stream of the operand's device and never
+synchronizes. A missing or unloadable library raises `KernelLibraryMissing` (a
+RuntimeError): there is no CPU or torch fallback behind these functions.
+"""
+
+import ctypes
+import threading
+from pathlib import Path
+
+import torch
+from torch import Tensor
+
+LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libkm_kernels.so"
+E4M3 = torch.float8_e4m3fn
+KM_BF16, KM_F16 = 0, 1
+KM_Q_INT8, KM_Q_E4M3 = 0, 1
+KERNEL_GEMM_MX, KERNEL_GEMM_FP8, KERNEL_WO_FWD, KERNEL_WO_DGRAD = 0, 1, 2, 3
+SCALES_ROWMAJOR, SCALES_PACKED = 0, 1
+_DTYPES = {torch.bfloat16: KM_BF16, torch.float16: KM_F16}
+_QFORMATS = {torch.int8: KM_Q_INT8, E4M3: KM_Q_E4M3}
+
+EXPORTS = (
+    "km_abi_version",
+    "km_last_error",
+    "km_quant_mx",
+    "km_scales_packed_bytes",
+    "km_scales_pack",
+    "km_quant_tensor",
+    "km_gemm_mx",
+    "km_gemm_fp8_tensor",
+    "km_wo_gemm_fwd",
+    "km_wo_gemm_dgrad",
+    "km_num_configs",
+    "km_config_desc",
+)
+
+_lock = threading.Lock()
+_lib: ctypes.CDLL | None = None
+
+
+class KernelLibraryMissing(RuntimeError):
+    """libkm_kernels.so is not built or cannot be loaded."""
+
+
+class KernelError(RuntimeError):
+    """A kernel entry point returned an error code (bad arguments or a failed launch)."""
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    c = ctypes
+    p, i64, i32 = c.c_void_p, c.c_int64, c.c_int
+    lib.km_abi_version.restype = i32
+    lib.km_last_error.restype = c.c_char_p
+    lib.km_quant_mx.argtypes = [p, i64, i64, i64, i64, i32, p, p, p, p]
+    lib.km_scales_packed_bytes.argtypes = [i64, i64]
+    lib.km_scales_pack.argtypes = [p, i64, i64, p, p]
+    lib.km_quant_tensor.argtypes = [p, i64, i64, i64, i64, i32, p, p, p, p]
+    lib.km_gemm_mx.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
+    lib.km_gemm_fp8_tensor.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
+    lib.km_wo_gemm_fwd.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
+    lib.km_wo_gemm_dgrad.argtypes = [p, p, p, p, i64, i64, i64, i32, i32, i32, p]
+    lib.km_num_configs.argtypes = [i32]
+    lib.km_config_desc.argtypes = [i32, i32, c.c_char_p, i32]
+    for name in EXPORTS:
+        if name not in ("km_last_error", "km_scales_packed_bytes"):
+            getattr(lib, name).restype = i32
+    lib.km_scales_packed_bytes.restype = i64
+
+
+def load() -> ctypes.CDLL:
+    """The loaded library (cached). Raises KernelLibraryMissing when it is not there."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            if not LIB_PATH.exists():
+                raise KernelLibraryMissing(
+                    f"{LIB_PATH} is not built; run `python -m kohakumosstrainer_amd.build` (needs hipcc)"
+                )
+            try:
+                lib = ctypes.CDLL(str(LIB_PATH))
+            except OSError as err:
+                raise KernelLibraryMissing(f"cannot load {LIB_PATH}: {err}") from err
+            missing = [n for n in EXPORTS if not hasattr(lib, n)]
+            if missing:
+                raise KernelLibraryMissing(f"{LIB_PATH} lacks {missing}")
+            _declare(lib)
+            _lib = lib
+    return _lib
+
+
+def available() -> str | None:
+    """None when the library loads, else why not."""
+    try:
+        load()
+    except KernelLibraryMissing as err:
+        return str(err)
+    return None
+
+
+def _check(code: int) -> None:
+    if code != 0:
+        raise KernelError(load().km_last_error().decode(errors="replace") or f"error {code}")
+
+
+def _stream(t: Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _on_gpu(*tensors: Tensor | None) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if t.device.type != "cuda":
+            raise ValueError(f"HIP kernels need device tensors, got {t.device}")
+        if dev is not None and t.device != dev:
+            raise ValueError(f"operands on different devices: {dev} and {t.device}")
+        dev = t.device
+    return dev
+
+
+def _dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"activation dtype {dtype} not in (bfloat16, float16)") from None
+
+
+# ---- quantizers -------------------------------------------------------------------------
+
+
+def packed_scale_bytes(rows: int, k: int) -> int:
+    """Size in bytes of the MFMA-packed scale copy of a [rows, k] operand (k % 128 == 0)."""
+    n = load().km_scales_packed_bytes(rows, k)
+    if n < 0:
+        raise ValueError(f"packed mx scales need K % 128 == 0, got K={k}")
+    return n
+
+
+def _new_packed(rows: int, k: int, device) -> Tensor:
+    n = packed_scale_bytes(rows, k)
+    # rows past the end of the last group of 128 are padding the GEMM may read: keep them zero
+    return (torch.zeros if rows % 128 else torch.empty)(n, device=device, dtype=torch.uint8)
+
+
+def quant_mx(x: Tensor, natural: bool = True, packed: bool = False):
+    """MXFP8 quantization of a 2-D bf16 / fp16 operand with any strides; blocks of 32 run
+    along the last axis (a transposed view `w.t()` takes the transposing kernel: column-wise
+    quantization). Returns `(q e4m3 [rows, K], scale uint8 [rows, K/32])`; with `packed`
+    the MFMA-packed scale copy (flat uint8, K % 128 == 0) is appended, and `natural=False`
+    returns None in place of the natural scales."""
+    if x.dim() != 2:
+        raise ValueError(f"fp8 operand must be 2-D, got {tuple(x.shape)}")
+    rows, k = x.shape
+    if k % 32:
+        raise ValueError(f"fp8 mx: K={k} is not a multiple of 32")
+    if not (natural or packed):
+        raise ValueError("quant_mx: ask for at least one scale layout")
+    _on_gpu(x)
+    q = torch.empty(rows, k, device=x.device, dtype=torch.uint8)
+    s = torch.empty(rows, k // 32, device=x.device, dtype=torch.uint8) if natural else None
+    sp = _new_packed(rows, k, x.device) if packed else None
+    with torch.cuda.device(x.device):
+        _check(
+            load().km_quant_mx(
+                x.data_ptr(), rows, k, x.stride(0), x.stride(1), _dtype_code(x.dtype), q.data_ptr(),
+                None if s is None else s.data_ptr(), None if sp is None else sp.data_ptr(), _stream(x),
+            )
+        )
+    return (q.view(E4M3), s, sp) if packed else (q.view(E4M3), s)
+
+
+def pack_scales(scale: Tensor) -> Tensor:
+    """The MFMA-packed copy of natural mx scales `[rows, K/32]` (K % 128 == 0)."""
+    if scale.dim() != 2 or scale.dtype != torch.uint8:
+        raise ValueError("mx scales must be a 2-D uint8 tensor")
+    _on_gpu(scale)
+    rows, blocks = scale.shape
+    scale = scale.contiguous()
+    out = _new_packed(rows, blocks * 32, scale.device)
+    with torch.cuda.device(scale.device):
+        _check(load().km_scales_pack(scale.data_ptr(), rows, blocks * 32, out.data_ptr(), _stream(scale)))
+    return out
+
+
+def quant_tensor(x: Tensor) -> tuple[Tensor, Tensor]:
+    """`(q e4m3 [rows, K], scale fp32 [1])` under the per-tensor recipe."""
+    if x.dim() != 2:
+        raise ValueError(f"fp8 operand must be 2-D, got {tuple(x.shape)}")
+    _on_gpu(x)
+    rows, k = x.shape
+    q = torch.empty(rows, k, device=x.device, dtype=torch.uint8)
+    s = torch.empty(1, device=x.device, dtype=torch.float32)
+    work = torch.empty(1, device=x.device, dtype=torch.int32)
+    with torch.cuda.device(x.device):
+        _check(load().km_quant_tensor(x.data_ptr(), rows, k, x.stride(0), x.stride(1), _dtype_code(x.dtype), q.data_ptr(), s.data_ptr(), work.data_ptr(), _stream(x)))
+    return q.view(E4M3), s
+
+
+# ---- GEMMs --------------------------------------------------------------------------------
+
+
+def _gemm_operands(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dtype):
+    if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
+        raise ValueError(f"GEMM operands must be [M, K] and [N, K], got {tuple(a.shape)} and {tuple(b.shape)}")
+    if a.dtype != E4M3 or b.dtype != E4M3:
+        raise ValueError(f"fp8 GEMM operands must be float8_e4m3fn, got {a.dtype} and {b.dtype}")
+    dev = _on_gpu(a, b, bias)
+    a, b = a.contiguous(), b.contiguous()
+    if bias is not None:
+        if bias.shape != (b.shape[0],):
+            raise ValueError(f"bias must be [{b.shape[0]}], got {tuple(bias.shape)}")
+        bias = bias.to(out_dtype).contiguous()
+    m, k = a.shape
+    c = torch.empty(m, b.shape[0], device=dev, dtype=out_dtype)
+    return a, b, bias, c, m, b.shape[0], k
+
+
+def gemm_mx(a: Tensor, a_scale: Tensor, b: Tensor, b_scale: Tensor, bias: Tensor | None, out_dtype: torch.dtype, config: int = 0, packed: bool = False) -> Tensor:
+    """`(a * 2^(a_scale-127)) (b * 2^(b_scale-127))^T + bias` -> `[M, N]` in `out_dtype`;
+    a `[M, K]`, b `[N, K]` e4m3, K a multiple of 128. Scales are uint8: natural
+    `[*, K/32]`, or with `packed` the flat MFMA-packed copies (`quant_mx(packed=True)`,
+    `pack_scales`)."""
+    a, b, bias, c, m, n, k = _gemm_operands(a, b, bias, out_dtype)
+    if a_scale.dtype != torch.uint8 or b_scale.dtype != torch.uint8:
+        raise ValueError("mx scales must be uint8 (biased E8M0)")
+    if packed:
+        if k % 128:
+            raise ValueError(f"packed mx scales need K % 128 == 0, got K={k}")
+        want = (packed_scale_bytes(m, k), packed_scale_bytes(n, k))
+        if (a_scale.numel(), b_scale.numel()) != want:
+            raise ValueError(f"packed mx scales must hold {want} bytes, got ({a_scale.numel()}, {b_scale.numel()})")
+    elif tuple(a_scale.shape) != (m, k // 32) or tuple(b_scale.shape) != (n, k // 32):
+        raise ValueError(f"mx scales must be [{m}, {k // 32}] and [{n}, {k // 32}], got {tuple(a_scale.shape)} and {tuple(b_scale.shape)}")
+    _on_gpu(a, a_scale, b_scale)
+    a_scale, b_scale = a_scale.contiguous(), b_scale.contiguous()
+    with torch.cuda.device(a.device):
+        _check(
+            load().km_gemm_mx(
+                a.data_ptr(), a_scale.data_ptr(), b.data_ptr(), b_scale.data_ptr(), None if bias is None else bias.data_ptr(),
+                c.data_ptr(), m, n, k, _dtype_code(out_dtype), SCALES_PACKED if packed else SCALES_ROWMAJOR, config, _stream(a),
+            )
+        )
+    return c
+
+
+def gemm_fp8_tensor(a: Tensor, sa: Tensor, b: Tensor, sb: Tensor, bias: Tensor | None, out_dtype: torch.dtype, config: int = 0) -> Tensor:
+    """`(a b^T) * sa * sb + bias`, sa / sb one-element fp32 device tensors."""
+    a, b, bias, c, m, n, k = _gemm_operands(a, b, bias, out_dtype)
+    if sa.numel() != 1 or sb.numel() != 1 or sa.dtype != torch.float32 or sb.dtype != torch.float32:
+        raise ValueError("per-tensor scales must be one-element fp32 tensors")
+    _on_gpu(a, sa, sb)
+    with torch.cuda.device(a.device):
+        _check(load().km_gemm_fp8_tensor(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), None if bias is None else bias.data_ptr(), c.data_ptr(), m, n, k, _dtype_code(out_dtype), config, _stream(a)))
+    return c
+
+
+def _wo_operands(x: Tensor, q: Tensor, scale: Tensor):
+    if x.dim() != 2 or q.dim() != 2:
+        raise ValueError(f"weight-only operands must be 2-D, got {tuple(x.shape)} and {tuple(q.shape)}")
+    if q.dtype not in _QFORMATS:
+        raise ValueError(f"weight codes must be int8 or float8_e4m3fn, got {q.dtype}")
+    if tuple(scale.shape) != (q.shape[0],):
+        raise ValueError(f"scale must be [{q.shape[0]}], got {tuple(scale.shape)}")
+    _on_gpu(x, q, scale)
+    return x.contiguous(), q.contiguous(), scale.to(torch.float32).contiguous()
+
+
+def wo_gemm_fwd(x: Tensor, q: Tensor, scale: Tensor, bias: Tensor | None, config: int = 0) -> Tensor:
+    """`(x @ q^T) * scale + bias` -> `[M, N]` in x's dtype; q `[N, K]` int8 / e4m3."""
+    x, q, scale = _wo_operands(x, q, scale)
+    if x.shape[1] != q.shape[1]:
+        raise ValueError(f"x is [M, {x.shape[1]}] but q is [N, {q.shape[1]}]")
+    m, k = x.shape
+    n = q.shape[0]
+    if bias is not None:
+        if bias.shape != (n,):
+            raise ValueError(f"bias must be [{n}], got {tuple(bias.shape)}")
+        _on_gpu(x, bias)
+        bias = bias.to(x.dtype).contiguous()
+    y = torch.empty(m, n, device=x.device, dtype=x.dtype)
+    with torch.cuda.device(x.device):
+        _check(load().km_wo_gemm_fwd(x.data_ptr(), q.data_ptr(), scale.data_ptr(), None if bias is None else bias.data_ptr(), y.data_ptr(), m, n, k, _QFORMATS[q.dtype], _dtype_code(x.dtype), config, _stream(x)))
+    return y
+
+
+def wo_gemm_dgrad(dy: Tensor, q: Tensor, scale: Tensor, config: int = 0) -> Tensor:
+    """`dy @ round(q * scale[:, None])` -> `[M, K]` in dy's dtype."""
+    dy, q, scale = _wo_operands(dy, q, scale)
+    if dy.shape[1] != q.shape[0]:
+        raise ValueError(f"dy is [M, {dy.shape[1]}] but q is [{q.shape[0]}, K]")
+    m, n = dy.shape
+    k = q.shape[1]
+    dx = torch.empty(m, k, device=dy.device, dtype=dy.dtype)
+    with torch.cuda.device(dy.device):
+        _check(load().km_wo_gemm_dgrad(dy.data_ptr(), q.data_ptr(), scale.data_ptr(), dx.data_ptr(), m, n, k, _QFORMATS[q.dtype], _dtype_code(dy.dtype), config, _stream(dy)))
+    return dx
+
+
+def configs(kernel: int) -> list[dict]:
+    """The tile configurations of one kernel family as dicts (`id` is the ABI config)."""
+    lib = load()
+    out = []
+    buf = ctypes.create_string_buffer(128)
+    for i in range(lib.km_num_configs(kernel)):
+        _check(lib.km_config_desc(kernel, i, buf, len(buf)))
+        row: dict = {"id": i}
+        for part in buf.value.decode().split(","):
+            key, _, val = part.partition("=")
+            row[key] = int(val) if val.lstrip("-").isdigit() else val
+        out.append(row)
+    return out

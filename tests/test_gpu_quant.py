@@ -1,0 +1,168 @@
+"""HIP quantizers against the CPU oracle, bit for bit, through the C ABI
+(`native.quant_mx` / `native.quant_tensor`). Mirrors reference
+`tests/kernels/quant/test_fp8.py:61-82` (bytes equal the eager reference, strided input)
+and adds the column-wise (transposed) case, an exhaustive bf16 sweep and the full-size
+`[16384, 3072]` operand with outliers."""
+
+import pytest
+import torch
+
+from kohakumosstrainer_amd import native
+from oracle import formats
+
+pytestmark = pytest.mark.gpu
+DTYPES = (torch.bfloat16, torch.float16)
+
+
+def u8(t):
+    return t.view(torch.uint8)
+
+
+def activations(m, k, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(m, k, generator=g) * torch.logspace(-3, 2, m)[:, None]
+    if m > 2:
+        x[1] = 0.0
+        x[2, : min(k, 32)] = torch.linspace(-1.75, 1.75, 32)[: min(k, 32)]
+    if m > 3 and k >= 64:
+        x[3, 32:64] = torch.linspace(-1.75, 1.75, 32) * (1 + 2.0**-7)
+    return x.to(dtype)
+
+
+def packed_reference(scale: torch.Tensor) -> torch.Tensor:
+    """The MFMA-packed copy of natural scales [rows, blocks] by its index formula: byte
+    (r, b) -> ((((b//4)*ceil(rows/128) + r//128)*16 + r%16)*4 + b%4)*8 + (r%128)//16."""
+    rows, blocks = scale.shape
+    groups = -(-rows // 128)
+    out = torch.zeros((blocks // 4) * groups * 512, dtype=torch.uint8)
+    r = torch.arange(rows)[:, None].expand(rows, blocks)
+    b = torch.arange(blocks)[None, :].expand(rows, blocks)
+    off = ((((b // 4) * groups + r // 128) * 16 + r % 16) * 4 + b % 4) * 8 + (r % 128) // 16
+    out[off.reshape(-1)] = scale.reshape(-1)
+    return out
+
+
+def check_mx(x_cpu: torch.Tensor, view=lambda t: t):
+    """Quantize `view(x)` on the GPU and with the oracle; bytes must be equal."""
+    xg = view(x_cpu.cuda())
+    q, s = native.quant_mx(xg)
+    rq, rs = formats.quantize(view(x_cpu), "mx", "act")
+    if xg.shape[1] % 128 == 0:
+        q2, s2, sp = native.quant_mx(xg, packed=True)
+        assert torch.equal(u8(q2), u8(q)) and torch.equal(s2, s)
+        assert torch.equal(sp.cpu(), packed_reference(rs)), "packed scale bytes"
+        _, none, sp3 = native.quant_mx(xg, natural=False, packed=True)
+        assert none is None and torch.equal(sp3, sp)
+        assert torch.equal(native.pack_scales(s), sp)
+    assert q.dtype == torch.float8_e4m3fn and s.dtype == torch.uint8
+    assert q.shape == rq.shape and s.shape == rs.shape
+    assert q.is_contiguous() and s.is_contiguous()
+    assert torch.equal(s.cpu(), rs), "scale bytes"
+    assert torch.equal(u8(q).cpu(), u8(rq)), "code bytes"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,k", [(300, 1024), (1, 32), (7, 96), (1000, 384), (33, 4096)])
+def test_mx_rows_bytes_equal_oracle(dtype, m, k):
+    check_mx(activations(m, k, dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,k", [(256, 64), (320, 200), (32, 8), (1024, 384), (96, 1000), (4096, 72)])
+def test_mx_cols_bytes_equal_oracle(dtype, m, k):
+    """Column-wise quantization: the operand is the transposed view of an [m, k] tensor."""
+    check_mx(activations(m, k, dtype, seed=3), view=lambda t: t.t())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_mx_strided_and_unaligned_views(dtype):
+    base = activations(130, 640, dtype, seed=5)
+    check_mx(base, view=lambda t: t[:, 64:576])  # row stride > K
+    check_mx(base, view=lambda t: t[3:, 32:96])  # aligned offset start
+    check_mx(base, view=lambda t: t[:, 1:65])  # 2-byte aligned only: generic kernel
+    check_mx(base, view=lambda t: t[::2, ::2][:, :160])  # both strides non-unit
+    check_mx(base, view=lambda t: t.t().contiguous().t())  # column-major storage
+    check_mx(base, view=lambda t: t[:96, :33].t())  # transposed, odd leading dimension
+
+
+def test_mx_every_finite_bf16_pattern():
+    x = torch.arange(65536, dtype=torch.int32).to(torch.uint16).view(torch.bfloat16)
+    x = x[torch.isfinite(x.float())]
+    x = x[: (x.numel() // 32) * 32]
+    for seed in range(4):
+        perm = torch.randperm(x.numel(), generator=torch.Generator().manual_seed(seed))
+        check_mx(x[perm].view(-1, 32 * (1 + seed % 2)))
+        check_mx(x[perm].view(32, -1), view=lambda t: t.t())
+
+
+def test_mx_zero_block_byte_and_sign_of_zero():
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    x[0, 0] = -0.0
+    x[1, :32] = torch.tensor([-1e-38, 1e-38] * 16, dtype=torch.bfloat16)
+    q, s = native.quant_mx(x.cuda())
+    assert s[0].tolist() == [19, 19] and s[2].tolist() == [19, 19]
+    assert u8(q)[0, 0].item() == 0x80 and u8(q)[0, 1].item() == 0
+    check_mx(x)
+
+
+def test_mx_nan_and_inf_elements():
+    x = activations(8, 128, torch.bfloat16)
+    x[0, 5] = float("inf")
+    x[4, 70] = float("nan")
+    q, s = native.quant_mx(x.cuda())
+    rq, rs = formats.quantize(x, "mx")
+    assert torch.equal(s.cpu(), rs) and torch.equal(u8(q).cpu(), u8(rq))
+
+
+def test_mx_argument_errors():
+    with pytest.raises(ValueError):
+        native.quant_mx(torch.zeros(4, 48, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ValueError):
+        native.quant_mx(torch.zeros(64, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ValueError):
+        native.quant_mx(torch.zeros(4, 64, dtype=torch.float32, device="cuda"))
+    with pytest.raises(ValueError):
+        native.quant_mx(torch.zeros(4, 64, dtype=torch.bfloat16))
+    q, s = native.quant_mx(torch.zeros(0, 64, dtype=torch.bfloat16, device="cuda"))
+    assert q.shape == (0, 64) and s.shape == (0, 2)
+
+
+def outlier_operand(m=16384, k=3072):
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(m, k, generator=g)
+    mask = torch.rand(m, k, generator=g) < 1e-3
+    x[mask] = (torch.randn(m, k, generator=g) * 50)[mask]
+    return x.to(torch.bfloat16)
+
+
+def test_mx_full_size_rows_and_cols_with_outliers():
+    """bf16 [16384, 3072] ~N(0,1) with 0.1 % entries +-N(0,50): row-wise and column-wise."""
+    x = outlier_operand()
+    check_mx(x)
+    check_mx(x, view=lambda t: t.t())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,k", [(300, 1024), (5, 7), (1, 1), (64, 200)])
+def test_tensor_recipe_bytes_equal_oracle(dtype, m, k):
+    x = activations(m, k, dtype, seed=7)
+    q, s = native.quant_tensor(x.cuda())
+    rq, rs = formats.quantize(x, "tensor")
+    assert s.dtype == torch.float32 and s.shape == (1,)
+    assert torch.equal(s.cpu(), rs)
+    assert torch.equal(u8(q).cpu(), u8(rq))
+    q2, s2 = native.quant_tensor(x.cuda().t())
+    rq2, rs2 = formats.quantize(x.t(), "tensor")
+    assert torch.equal(s2.cpu(), rs2) and torch.equal(u8(q2).cpu(), u8(rq2))
+
+
+def test_tensor_recipe_all_zero_and_weight_like():
+    z = torch.zeros(16, 64, dtype=torch.bfloat16)
+    q, s = native.quant_tensor(z.cuda())
+    rq, rs = formats.quantize(z, "tensor")
+    assert torch.equal(s.cpu(), rs) and torch.equal(u8(q).cpu(), u8(rq))
+    g = torch.Generator().manual_seed(1)
+    w = (torch.randn(1024, 768, generator=g) * 0.02).to(torch.bfloat16)
+    q, s = native.quant_tensor(w.cuda())
+    rq, rs = formats.quantize(w, "tensor")
+    assert torch.equal(s.cpu(), rs) and torch.equal(u8(q).cpu(), u8(rq))
