@@ -9,12 +9,14 @@
 // the per-tensor recipe; the shared epilogue _store :40-49).
 //
 // Shape of the kernel. A workgroup of four wavefronts owns a BM x BN tile of C and walks K in
-// steps of 128 bytes. Per step the A (BM x 128 B) and B (BN x 128 B) slabs live in one of two
-// static LDS stages, filled by direct-to-LDS buffer loads (no staging registers): the loads of
-// step k+1 are issued at the top of step k into the other stage and waited for just before
-// the last MFMA group of step k, where the one barrier of the step sits; the fragments of
-// step k+1 are then read during that last group, so the MFMA pipe has work across the step
-// boundary. Each wavefront computes a (BM/2) x (BN/2) sub-tile as 16x16 MFMA tiles. The
+// steps of 128 bytes. Per step the A (BM x 128 B) and B (BN x 128 B) slabs live in two pairs
+// of static LDS buffers, filled by direct-to-LDS buffer loads (no staging registers). The A
+// fragments of a step are read into registers during the last MFMA group of the step before,
+// so an A buffer is free a whole step early: at the top of step k the loads of B(k+1) and then
+// of A(k+2) are issued, and just before the last MFMA group of step k the wavefront waits
+// only for B(k+1) (vmcnt counts in order), passes the barrier and reads the first fragments of
+// step k+1. The A(k+2) loads stay in flight across that barrier, so the fetch stream never
+// drains and the MFMA pipe has work across the step boundary. Each wavefront computes a (BM/2) x (BN/2) sub-tile as 16x16 MFMA tiles. The
 // MFMA's "A" operand (rows of the 16x16 result) is fed from B (output columns n) and its "B"
 // operand from A (tokens m), so a lane ends up with 4 consecutive n of one m and stores 8
 // bytes of bf16. Rows past M / N are fetched through buffer descriptors whose range check
@@ -58,16 +60,20 @@ __device__ __forceinline__ int slab_offset(int row, int chunk) {
   return (((row >> 4) * 8 + (row & 7)) << 8) + (((row >> 3) & 1) << 7) + ((chunk ^ (row & 7)) << 4);
 }
 
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+// two fp32 -> two 16-bit values in one register, round to nearest even (one v_cvt_pk_* each)
 template <int OUT>
 __device__ __forceinline__ uint32_t pack2(float a, float b);
 template <>
 __device__ __forceinline__ uint32_t pack2<KM_BF16>(float a, float b) {
-  return f32_to_bf16_bits(a) | (f32_to_bf16_bits(b) << 16);
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{a, b}), bf16x2));
 }
 template <>
 __device__ __forceinline__ uint32_t pack2<KM_F16>(float a, float b) {
-  _Float16 x = (_Float16)a, y = (_Float16)b;
-  return (uint32_t)__builtin_bit_cast(uint16_t, x) | ((uint32_t)__builtin_bit_cast(uint16_t, y) << 16);
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{a, b}), f16x2));
 }
 template <int OUT>
 __device__ __forceinline__ float unpack1(uint32_t h);
@@ -140,7 +146,8 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 // s_waitcnt immediates (gfx9 encoding: vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8])
 constexpr int kWaitVm0 = 0x0F70;         // vmcnt(0)
-constexpr int kWaitVm0Lgkm0 = 0x0070;    // vmcnt(0) lgkmcnt(0)
+constexpr int kWaitLgkm0 = 0xC07F;       // lgkmcnt(0)
+constexpr int wait_vm_lgkm0(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070; }  // vmcnt(n) lgkmcnt(0)
 
 template <int BM, int BN, bool MX, bool SCALE_KM, int OUT>
 __global__ __launch_bounds__(256) void gemm_fp8_kernel(
@@ -151,11 +158,14 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
   constexpr int WTM = BM / 2, WTN = BN / 2;
   constexpr int TM = WTM / 16, TN = WTN / 16;
   constexpr int A_BYTES = BM * kStepBytes, B_BYTES = BN * kStepBytes;
-  constexpr int STAGE = A_BYTES + B_BYTES;
   constexpr int A_LD = BM / 32, B_LD = BN / 32;  // 32 rows (4 KiB) per pass of 256 lanes
+  constexpr int kWaitAllButA = wait_vm_lgkm0(A_LD);  // all but the A_LD newest loads done
   static_assert(BM % 32 == 0 && BN % 32 == 0 && TM >= 1 && TN >= 2, "tile");
-  __shared__ __attribute__((aligned(1024))) uint8_t stage0[STAGE];
-  __shared__ __attribute__((aligned(1024))) uint8_t stage1[STAGE];
+  static_assert(TM * (TN - 1) >= BM / 32 + BN / 32, "every fetch pass needs its own MFMA slot");
+  __shared__ __attribute__((aligned(1024))) uint8_t a_buf0[A_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t a_buf1[A_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t b_buf0[B_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t b_buf1[B_BYTES];
 
   int tile_m, tile_n;
   tile_of(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, tile_n);
@@ -231,16 +241,24 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
   int wscale[2][WS], xscale[2][XS];
   uint32_t wraw[WS], xraw[XS];
 
-  auto dma = [&](uint8_t* stage, int ks) __attribute__((always_inline)) {
+  // one 4 KiB pass (32 rows) of a slab: each wavefront moves 1 KiB with one instruction
+  auto dma_a_pass = [&](uint8_t* buf, int koff, int i) __attribute__((always_inline)) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(buf + i * 4096 + wave * 1024), 16,
+                                             ld_voff + i * pass_stride, koff, 0, 0);
+  };
+  auto dma_b_pass = [&](uint8_t* buf, int koff, int i) __attribute__((always_inline)) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(buf + i * 4096 + wave * 1024), 16,
+                                             ld_voff + i * pass_stride, koff, 0, 0);
+  };
+  auto dma_a = [&](uint8_t* buf, int ks) __attribute__((always_inline)) {
     const int koff = __builtin_amdgcn_readfirstlane(ks * kStepBytes);
 #pragma unroll
-    for (int i = 0; i < A_LD; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(stage + i * 4096 + wave * 1024), 16,
-                                               ld_voff + i * pass_stride, koff, 0, 0);
+    for (int i = 0; i < A_LD; ++i) dma_a_pass(buf, koff, i);
+  };
+  auto dma_b = [&](uint8_t* buf, int ks) __attribute__((always_inline)) {
+    const int koff = __builtin_amdgcn_readfirstlane(ks * kStepBytes);
 #pragma unroll
-    for (int i = 0; i < B_LD; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(stage + A_BYTES + i * 4096 + wave * 1024), 16,
-                                               ld_voff + i * pass_stride, koff, 0, 0);
+    for (int i = 0; i < B_LD; ++i) dma_b_pass(buf, koff, i);
   };
   auto scale_fetch = [&](int ks) __attribute__((always_inline)) {
     if constexpr (MX) {
@@ -287,42 +305,74 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
     const v4i hi = *reinterpret_cast<const v4i*>(slab + slab_offset(row, g + 4));
     return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
-  // One K step out of `cur` with scale set P. Step ks+1 (clamped to the last one) is fetched
-  // into `nxt` meanwhile; its first fragments are read after the barrier, during the last MFMA
-  // group (each fragment register is reloaded one MFMA after the last MFMA that read it), and
-  // its scales are committed to set P^1.
-  auto step = [&](uint8_t* cur, uint8_t* nxt, int ks, auto set_tag) __attribute__((always_inline)) {
+  // One K step with parity P: A(k) is already in registers, B(k) is in b_cur. Fetches B(k+1)
+  // into b_nxt and A(k+2) into a_cur (its A(k) was consumed during the step before; the
+  // barrier at the top makes sure by every wavefront), multiplies, waits for B(k+1) only,
+  // and reads the first fragments of step k+1 (A(k+1) from a_nxt was issued a step earlier)
+  // during the last MFMA group; each fragment register is reloaded one MFMA after the last
+  // MFMA that read it. The scales of step k+1 are committed to set P^1.
+  //
+  // The fetch instructions are spread between the MFMAs of the first TN-1 groups (B passes
+  // over the first third, A passes over the rest): a wavefront that queues them back to back
+  // blocks on the address unit it shares with the other three and issues no MFMA meanwhile.
+  constexpr int kWindow = TM * (TN - 1);           // MFMAs before the last group
+  constexpr int kBWindow = kWindow / 3 > B_LD ? kWindow / 3 : B_LD;
+  auto step = [&](uint8_t* a_cur, uint8_t* a_nxt, uint8_t* b_cur, uint8_t* b_nxt, int ks, auto set_tag)
+                  __attribute__((always_inline)) {
     constexpr int P = decltype(set_tag)::value;
     const int next = min(ks + 1, nk - 1);
-    dma(nxt, next);
+    const int koff_b = __builtin_amdgcn_readfirstlane(next * kStepBytes);
+    const int koff_a = __builtin_amdgcn_readfirstlane(min(ks + 2, nk - 1) * kStepBytes);
+    __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+    __syncthreads();  // every wavefront has read its A(k) fragments out of a_cur
     scale_fetch(next);
-    __builtin_amdgcn_sched_barrier(0);  // keep the fetches at the top of the step
+    __builtin_amdgcn_sched_barrier(0);
     static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
       constexpr int t = decltype(t_tag)::value;
       v8i wnext;
       if constexpr (t + 1 < TN) {
-        wnext = fragment(cur + A_BYTES, wn + (t + 1) * 16 + r16);
+        wnext = fragment(b_cur, wn + (t + 1) * 16 + r16);
       } else {
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
+        __builtin_amdgcn_s_waitcnt(kWaitAllButA);  // B(k+1), scales(k+1) (and A(k+1)) landed
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        wnext = fragment(nxt + A_BYTES, wn + r16);
+        wnext = fragment(b_nxt, wn + r16);
       }
       static_for<TM>([&](auto j_tag) __attribute__((always_inline)) {
         constexpr int j = decltype(j_tag)::value;
+        constexpr int q = t * TM + j;  // position in the step's MFMA sequence
         if constexpr (SCALE_KM)
           mfma_acc<t, j>(acc[t][j], wcur, xf[j], wscale[P][(t >> 2) % WS], xscale[P][(j >> 2) % XS]);
         else
           mfma_acc<0, 0>(acc[t][j], wcur, xf[j], wscale[P][t % WS], xscale[P][j % XS]);
+        if constexpr (t + 1 < TN) {
+          // B pass i goes after MFMA i*kBWindow/B_LD, A pass i after kBWindow + i*(kWindow-kBWindow)/A_LD
+          static_for<B_LD>([&](auto i_tag) __attribute__((always_inline)) {
+            constexpr int i = decltype(i_tag)::value;
+            if constexpr (q == i * kBWindow / B_LD) {
+              __builtin_amdgcn_sched_barrier(0);
+              dma_b_pass(b_nxt, koff_b, i);
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          });
+          static_for<A_LD>([&](auto i_tag) __attribute__((always_inline)) {
+            constexpr int i = decltype(i_tag)::value;
+            if constexpr (q == kBWindow + i * (kWindow - kBWindow) / A_LD) {
+              __builtin_amdgcn_sched_barrier(0);
+              dma_a_pass(a_cur, koff_a, i);
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          });
+        }
         if constexpr (t + 1 == TN && j >= 1) {
           __builtin_amdgcn_sched_barrier(0);
-          xf[j - 1] = fragment(nxt, wm + (j - 1) * 16 + r16);
+          xf[j - 1] = fragment(a_nxt, wm + (j - 1) * 16 + r16);
         }
       });
       if constexpr (t + 1 == TN) {
         __builtin_amdgcn_sched_barrier(0);
-        xf[TM - 1] = fragment(nxt, wm + (TM - 1) * 16 + r16);
+        xf[TM - 1] = fragment(a_nxt, wm + (TM - 1) * 16 + r16);
       }
       wcur = wnext;
     });
@@ -332,22 +382,25 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
   using set0_t = std::integral_constant<int, 0>;
   using set1_t = std::integral_constant<int, 1>;
 
-  // prologue: step 0 into stage0, scale set 0
-  dma(stage0, 0);
+  // prologue: A(0), B(0), A(1) and the scales of step 0
+  dma_a(a_buf0, 0);
+  dma_b(b_buf0, 0);
   scale_fetch(0);
+  dma_a(a_buf1, min(1, nk - 1));
   __builtin_amdgcn_s_waitcnt(kWaitVm0);
   __syncthreads();
   scale_commit(set0_t{}, 0xFFFFFFFFu);
 #pragma unroll
-  for (int j = 0; j < TM; ++j) xf[j] = fragment(stage0, wm + j * 16 + r16);
-  wcur = fragment(stage0 + A_BYTES, wn + r16);
+  for (int j = 0; j < TM; ++j) xf[j] = fragment(a_buf0, wm + j * 16 + r16);
+  wcur = fragment(b_buf0, wn + r16);
 
-  // two steps per trip, one per stage; an odd step count is padded with a zero-scaled step
+  // two steps per trip, one per buffer parity; an odd step count is padded with a zero-scaled step
   const int nsteps = (nk + 1) & ~1;
   for (int ks = 0; ks < nsteps; ks += 2) {
-    step(stage0, stage1, ks, set0_t{});
-    step(stage1, stage0, ks + 1, set1_t{});
+    step(a_buf0, a_buf1, b_buf0, b_buf1, ks, set0_t{});
+    step(a_buf1, a_buf0, b_buf1, b_buf0, ks + 1, set1_t{});
   }
+  __builtin_amdgcn_s_waitcnt(kWaitVm0);  // the last (clamped) A prefetch must land before LDS is reused
 
   // the MFMAs above are opaque to the compiler's hazard handling: give the last ones time to
   // retire before the accumulators are read
@@ -358,12 +411,65 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
   // epilogue: lane holds C[m][n .. n+3] for m = m0+wm+j*16+r16, n = n0+wn+t*16+4*g
   float post = 1.0f;
   if constexpr (!MX) post = sa[0] * sb[0];
+  const bool has_bias = bias != nullptr;
+  if (m0 + BM <= M && n0 + BN <= N && (N & 7) == 0) {
+    // Interior tile. A lane holds 4 consecutive n of 16 different rows per MFMA tile; storing
+    // that directly makes 32-byte write requests. Instead each wavefront transposes its
+    // sub-tile through LDS (idle now), 64 rows at a time: 8-byte LDS writes in the MFMA
+    // layout, 16-byte LDS reads along rows, 16-byte global stores that cover whole
+    // WTN*2-byte row segments (full 128-byte lines).
+    constexpr int RP = WTN * 2 + 32;            // LDS row pitch in bytes (pad spreads banks)
+    constexpr int kMinBuf = A_BYTES < B_BYTES ? A_BYTES : B_BYTES;
+    constexpr int HM0 = TM < 4 ? TM : 4;        // MFMA tiles (of 16 rows) per pass, halved until
+    constexpr int HM = HM0 * 16 * RP <= kMinBuf ? HM0 : (HM0 / 2) * 16 * RP <= kMinBuf ? HM0 / 2 : 1;  // it fits a buffer
+    constexpr int LPR = WTN * 2 / 16;           // lanes per row on the read side
+    constexpr int RPI = 64 / LPR;               // rows per read instruction
+    static_assert(HM * 16 * RP <= A_BYTES && HM * 16 * RP <= B_BYTES, "epilogue staging: one buffer per wavefront");
+    __syncthreads();  // every wavefront is done reading fragments
+    uint8_t* region = wave == 0 ? a_buf0 : wave == 1 ? a_buf1 : wave == 2 ? b_buf0 : b_buf1;
+    const uint16_t* bias_lane = bias + (has_bias ? n0 + wn + 4 * g : 0);
+    float bv[TN][4];
+    static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
+      constexpr int t = decltype(t_tag)::value;
+      bv[t][0] = bv[t][1] = bv[t][2] = bv[t][3] = 0.f;
+      if (has_bias) {
+        const uint2 braw = *reinterpret_cast<const uint2*>(bias_lane + t * 16);
+        bv[t][0] = unpack1<OUT>(braw.x & 0xFFFFu); bv[t][1] = unpack1<OUT>(braw.x >> 16);
+        bv[t][2] = unpack1<OUT>(braw.y & 0xFFFFu); bv[t][3] = unpack1<OUT>(braw.y >> 16);
+      }
+    });
+    uint8_t* out_base = reinterpret_cast<uint8_t*>(C) + ((size_t)(m0 + wm) * N + n0 + wn) * 2;
+    const int rd_row = lane / LPR, rd_col = (lane % LPR) * 16;
+    static_for<TM / HM>([&](auto p_tag) __attribute__((always_inline)) {
+      constexpr int pass = decltype(p_tag)::value;
+      static_for<HM>([&](auto j_tag) __attribute__((always_inline)) {
+        constexpr int jj = decltype(j_tag)::value;
+        constexpr int j = pass * HM + jj;
+        static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
+          constexpr int t = decltype(t_tag)::value;
+          float o[4];
+#pragma unroll
+          for (int v = 0; v < 4; ++v) o[v] = MX ? acc[t][j][v] + bv[t][v] : acc[t][j][v] * post + bv[t][v];
+          *reinterpret_cast<uint2*>(region + (jj * 16 + r16) * RP + (t * 16 + 4 * g) * 2) =
+              make_uint2(pack2<OUT>(o[0], o[1]), pack2<OUT>(o[2], o[3]));
+        });
+      });
+      // only this wavefront touches its region: LDS operations of one wavefront stay in order
+      static_for<HM * 16 / RPI>([&](auto i_tag) __attribute__((always_inline)) {
+        constexpr int i = decltype(i_tag)::value;
+        const int row = i * RPI + rd_row;  // within the pass
+        const uint4 v = *reinterpret_cast<const uint4*>(region + row * RP + rd_col);
+        *reinterpret_cast<uint4*>(out_base + (size_t)(pass * HM * 16 + row) * N * 2 + rd_col) = v;
+      });
+    });
+    return;
+  }
   const bool vec_ok = (N & 3) == 0;
 #pragma unroll
   for (int t = 0; t < TN; ++t) {
     const int n = n0 + wn + t * 16 + 4 * g;
     float bv[4] = {0.f, 0.f, 0.f, 0.f};
-    if (bias != nullptr) {
+    if (has_bias) {
 #pragma unroll
       for (int v = 0; v < 4; ++v)
         if (n + v < N) bv[v] = unpack1<OUT>(bias[n + v]);
