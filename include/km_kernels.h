@@ -90,9 +90,12 @@ int km_wo_gemm_fwd(const void *x, const void *q, const float *scale, const void 
 
 /* Weight-only input gradient: dx[M,K] = dy[M,N] @ round_dtype(q[N,K] * scale[N]); the scaled
  * weight tile is rounded once to the activation dtype, as dequantize-then-matmul does.
+ * q_t_workspace is N*K bytes of device memory the call owns while it runs (the codes are
+ * transposed into it so that the contraction axis N becomes contiguous).
  * Replaces Triton _dgrad_kernel (backends/triton/quant.py:80-129). */
-int km_wo_gemm_dgrad(const void *dy, const void *q, const float *scale, void *dx, int64_t M,
-                     int64_t N, int64_t K, int q_format, int dtype, int config, void *stream);
+int km_wo_gemm_dgrad(const void *dy, const void *q, const float *scale, void *dx,
+                     void *q_t_workspace, int64_t M, int64_t N, int64_t K, int q_format, int dtype,
+                     int config, void *stream);
 
 /* Tile configurations per kernel, for the host-side tuning table (the reference enumerates its
  * Triton tiles in backends/triton/fp8/linear.py:39-75 and backends/triton/quant.py:132-141). */

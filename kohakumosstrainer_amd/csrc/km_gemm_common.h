@@ -1,0 +1,190 @@
+// Machinery shared by the GEMM kernels: the swizzled LDS slab layout, the work-group to tile
+// map, 16-bit packing, compile-time loops and the epilogue that writes a wavefront's
+// accumulators through an LDS transpose.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+#include <utility>
+
+#include "km_internal.h"
+#include "km_numeric.h"
+
+namespace km {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kStepBytes = 128;  // K bytes per step (= K elements, e4m3)
+
+__device__ __forceinline__ int slab_offset(int row, int chunk) {
+  return (((row >> 4) * 8 + (row & 7)) << 8) + (((row >> 3) & 1) << 7) + ((chunk ^ (row & 7)) << 4);
+}
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+// two fp32 -> two 16-bit values in one register, round to nearest even (one v_cvt_pk_* each)
+template <int OUT>
+__device__ __forceinline__ uint32_t pack2(float a, float b);
+template <>
+__device__ __forceinline__ uint32_t pack2<KM_BF16>(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{a, b}), bf16x2));
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<KM_F16>(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{a, b}), f16x2));
+}
+template <int OUT>
+__device__ __forceinline__ float unpack1(uint32_t h);
+template <>
+__device__ __forceinline__ float unpack1<KM_BF16>(uint32_t h) { return bits_f32(h << 16); }
+template <>
+__device__ __forceinline__ float unpack1<KM_F16>(uint32_t h) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+
+// Work-group id -> (tile_m, tile_n). Work-groups are dealt round-robin to the 8 XCDs, each
+// with its own L2; first give every XCD a contiguous run of tiles, then walk that run in
+// bands of kGroupM row-tiles so that neighbours in time share A rows and B rows in L2.
+constexpr int kXcds = 8;
+constexpr int kGroupM = 8;
+__device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  const int xcd = pid % kXcds, local = pid / kXcds;
+  const int tall = total / kXcds, rem = total % kXcds;
+  int p = xcd < rem ? xcd * (tall + 1) + local : rem * (tall + 1) + (xcd - rem) * tall + local;
+  const int per_group = kGroupM * tiles_n;
+  const int first_m = (p / per_group) * kGroupM;
+  const int group_m = min(tiles_m - first_m, kGroupM);
+  const int in_group = p % per_group;
+  tm = first_m + in_group % group_m;
+  tn = in_group / group_m;
+}
+
+// compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// s_waitcnt immediates (gfx9 encoding: vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8])
+constexpr int kWaitVm0 = 0x0F70;         // vmcnt(0)
+constexpr int kWaitLgkm0 = 0xC07F;       // lgkmcnt(0)
+constexpr int wait_vm_lgkm0(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070; }  // vmcnt(n) lgkmcnt(0)
+
+// Epilogue of a 2 x 2 wavefront grid over a BM x BN tile of 16x16 MFMA tiles whose rows are
+// output columns: lane (r16 = lane%16, g = lane/16) of tile (t, j) holds
+// C[m0+wm+j*16+r16][n0+wn+t*16+4g .. +3]. Computes acc * post * col_scale[n] + bias[n] in fp32,
+// rounds once to the 16-bit output type. `bufs` are four LDS buffers of at least
+// `buf_bytes` each, free for staging (one per wavefront).
+template <int BM, int BN, int OUT, bool SCALED>
+__device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float post, const float* __restrict__ col_scale,
+                                           const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N,
+                                           int m0, int n0, uint8_t* buf0, uint8_t* buf1, uint8_t* buf2, uint8_t* buf3) {
+  constexpr int WTM = BM / 2, WTN = BN / 2, TM = WTM / 16, TN = WTN / 16;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = (wave >> 1) * WTM, wn = (wave & 1) * WTN;
+  const int r16 = lane & 15, g = lane >> 4;
+  const bool has_bias = bias != nullptr;
+  auto value = [&](float a, float cs, float b) __attribute__((always_inline)) {
+    if constexpr (SCALED) return a * (post * cs) + b;
+    else return a + b;
+  };
+  if (m0 + BM <= M && n0 + BN <= N && (N & 7) == 0) {
+    // Interior tile. A lane holds 4 consecutive n of 16 different rows per MFMA tile; storing
+    // that directly makes 32-byte write requests. Instead each wavefront transposes its
+    // sub-tile through LDS (idle now), 64 rows at a time: 8-byte LDS writes in the MFMA
+    // layout, 16-byte LDS reads along rows, 16-byte global stores that cover whole
+    // WTN*2-byte row segments (full 128-byte lines).
+    constexpr int RP = WTN * 2 + 32;            // LDS row pitch in bytes (pad spreads banks)
+    constexpr int kMinBuf = (BM < BN ? BM : BN) * 128;
+    constexpr int HM0 = TM < 4 ? TM : 4;        // MFMA tiles (of 16 rows) per pass, halved until
+    constexpr int HM = HM0 * 16 * RP <= kMinBuf ? HM0 : (HM0 / 2) * 16 * RP <= kMinBuf ? HM0 / 2 : 1;  // it fits a buffer
+    constexpr int LPR = WTN * 2 / 16;           // lanes per row on the read side
+    constexpr int RPI = 64 / LPR;               // rows per read instruction
+    static_assert(HM * 16 * RP <= kMinBuf, "epilogue staging: one buffer per wavefront");
+    __syncthreads();  // every wavefront is done reading fragments
+    uint8_t* region = wave == 0 ? buf0 : wave == 1 ? buf1 : wave == 2 ? buf2 : buf3;
+    const uint16_t* bias_lane = bias + (has_bias ? n0 + wn + 4 * g : 0);
+    float bv[TN][4], cs[TN][4];
+    static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
+      constexpr int t = decltype(t_tag)::value;
+      bv[t][0] = bv[t][1] = bv[t][2] = bv[t][3] = 0.f;
+      cs[t][0] = cs[t][1] = cs[t][2] = cs[t][3] = 1.f;
+      if (col_scale != nullptr) {
+        const float4 c4 = *reinterpret_cast<const float4*>(col_scale + n0 + wn + 4 * g + t * 16);
+        cs[t][0] = c4.x; cs[t][1] = c4.y; cs[t][2] = c4.z; cs[t][3] = c4.w;
+      }
+      if (has_bias) {
+        const uint2 braw = *reinterpret_cast<const uint2*>(bias_lane + t * 16);
+        bv[t][0] = unpack1<OUT>(braw.x & 0xFFFFu); bv[t][1] = unpack1<OUT>(braw.x >> 16);
+        bv[t][2] = unpack1<OUT>(braw.y & 0xFFFFu); bv[t][3] = unpack1<OUT>(braw.y >> 16);
+      }
+    });
+    uint8_t* out_base = reinterpret_cast<uint8_t*>(C) + ((size_t)(m0 + wm) * N + n0 + wn) * 2;
+    const int rd_row = lane / LPR, rd_col = (lane % LPR) * 16;
+    static_for<TM / HM>([&](auto p_tag) __attribute__((always_inline)) {
+      constexpr int pass = decltype(p_tag)::value;
+      static_for<HM>([&](auto j_tag) __attribute__((always_inline)) {
+        constexpr int jj = decltype(j_tag)::value;
+        constexpr int j = pass * HM + jj;
+        static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
+          constexpr int t = decltype(t_tag)::value;
+          float o[4];
+#pragma unroll
+          for (int v = 0; v < 4; ++v) o[v] = value(acc[t][j][v], cs[t][v], bv[t][v]);
+          *reinterpret_cast<uint2*>(region + (jj * 16 + r16) * RP + (t * 16 + 4 * g) * 2) =
+              make_uint2(pack2<OUT>(o[0], o[1]), pack2<OUT>(o[2], o[3]));
+        });
+      });
+      // only this wavefront touches its region: LDS operations of one wavefront stay in order
+      static_for<HM * 16 / RPI>([&](auto i_tag) __attribute__((always_inline)) {
+        constexpr int i = decltype(i_tag)::value;
+        const int row = i * RPI + rd_row;  // within the pass
+        const uint4 v = *reinterpret_cast<const uint4*>(region + row * RP + rd_col);
+        *reinterpret_cast<uint4*>(out_base + (size_t)(pass * HM * 16 + row) * N * 2 + rd_col) = v;
+      });
+    });
+    return;
+  }
+  const bool vec_ok = (N & 3) == 0;
+#pragma unroll
+  for (int t = 0; t < TN; ++t) {
+    const int n = n0 + wn + t * 16 + 4 * g;
+    float bv[4] = {0.f, 0.f, 0.f, 0.f}, cs[4] = {1.f, 1.f, 1.f, 1.f};
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      if (has_bias && n + v < N) bv[v] = unpack1<OUT>(bias[n + v]);
+      if (col_scale != nullptr && n + v < N) cs[v] = col_scale[n + v];
+    }
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      const int m = m0 + wm + j * 16 + r16;
+      if (m >= M || n >= N) continue;
+      float o[4];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) o[v] = value(acc[t][j][v], cs[v], bv[v]);
+      uint16_t* dst = C + (size_t)m * N + n;
+      if (vec_ok && n + 3 < N) {
+        *reinterpret_cast<uint2*>(dst) = make_uint2(pack2<OUT>(o[0], o[1]), pack2<OUT>(o[2], o[3]));
+      } else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (n + v < N) dst[v] = (uint16_t)(pack2<OUT>(o[v], 0.f) & 0xFFFFu);
+      }
+    }
+  }
+}
+
+}  // namespace km

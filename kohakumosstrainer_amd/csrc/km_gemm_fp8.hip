@@ -38,79 +38,11 @@
 // the fragment reads (16 lanes = 16 rows at one chunk) touch every bank once. A direct-to-LDS
 // load writes lane i of a wavefront at base + 16*i, so the swizzle is applied on the global
 // side: lane i fetches the chunk whose slot is i & 7.
-#include <hip/hip_runtime.h>
-#include <stdint.h>
 #include <stdio.h>
 
-#include <type_traits>
-#include <utility>
-
-#include "km_internal.h"
-#include "km_numeric.h"
+#include "km_gemm_common.h"
 
 namespace km {
-
-typedef int v8i __attribute__((ext_vector_type(8)));
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef float v4f __attribute__((ext_vector_type(4)));
-
-constexpr int kStepBytes = 128;  // K bytes per step (= K elements, e4m3)
-
-__device__ __forceinline__ int slab_offset(int row, int chunk) {
-  return (((row >> 4) * 8 + (row & 7)) << 8) + (((row >> 3) & 1) << 7) + ((chunk ^ (row & 7)) << 4);
-}
-
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-
-// two fp32 -> two 16-bit values in one register, round to nearest even (one v_cvt_pk_* each)
-template <int OUT>
-__device__ __forceinline__ uint32_t pack2(float a, float b);
-template <>
-__device__ __forceinline__ uint32_t pack2<KM_BF16>(float a, float b) {
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{a, b}), bf16x2));
-}
-template <>
-__device__ __forceinline__ uint32_t pack2<KM_F16>(float a, float b) {
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{a, b}), f16x2));
-}
-template <int OUT>
-__device__ __forceinline__ float unpack1(uint32_t h);
-template <>
-__device__ __forceinline__ float unpack1<KM_BF16>(uint32_t h) { return bits_f32(h << 16); }
-template <>
-__device__ __forceinline__ float unpack1<KM_F16>(uint32_t h) {
-  return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
-}
-
-// Work-group id -> (tile_m, tile_n). Work-groups are dealt round-robin to the 8 XCDs, each
-// with its own L2; first give every XCD a contiguous run of tiles, then walk that run in
-// bands of kGroupM row-tiles so that neighbours in time share A rows and B rows in L2.
-constexpr int kXcds = 8;
-constexpr int kGroupM = 8;
-__device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
-  const int total = tiles_m * tiles_n;
-  const int xcd = pid % kXcds, local = pid / kXcds;
-  const int tall = total / kXcds, rem = total % kXcds;
-  int p = xcd < rem ? xcd * (tall + 1) + local : rem * (tall + 1) + (xcd - rem) * tall + local;
-  const int per_group = kGroupM * tiles_n;
-  const int first_m = (p / per_group) * kGroupM;
-  const int group_m = min(tiles_m - first_m, kGroupM);
-  const int in_group = p % per_group;
-  tm = first_m + in_group % group_m;
-  tn = in_group / group_m;
-}
-
-// compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
-template <class F, int... Is>
-__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
-  (f(std::integral_constant<int, Is>{}), ...);
-}
-template <int N, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-  static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
-}
 
 // c += A(16x128) * B(128x16) with block scales, accumulating in place: the accumulator is an
 // AGPR tuple tied as input and output ("+a"), which keeps all 64 tiles of a wavefront resident
@@ -141,13 +73,6 @@ __device__ __forceinline__ void mfma_acc(v4f& c, const v8i& a, const v8i& b, int
   else KM_MFMA_ASM(1, 1, 1, 1);
 }
 #undef KM_MFMA_ASM
-
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-
-// s_waitcnt immediates (gfx9 encoding: vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8])
-constexpr int kWaitVm0 = 0x0F70;         // vmcnt(0)
-constexpr int kWaitLgkm0 = 0xC07F;       // lgkmcnt(0)
-constexpr int wait_vm_lgkm0(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070; }  // vmcnt(n) lgkmcnt(0)
 
 template <int BM, int BN, bool MX, bool SCALE_KM, int OUT>
 __global__ __launch_bounds__(256) void gemm_fp8_kernel(
@@ -408,89 +333,10 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
 
-  // epilogue: lane holds C[m][n .. n+3] for m = m0+wm+j*16+r16, n = n0+wn+t*16+4*g
+  // epilogue: bias (and the per-tensor scales) on the fp32 accumulator, one rounding
   float post = 1.0f;
   if constexpr (!MX) post = sa[0] * sb[0];
-  const bool has_bias = bias != nullptr;
-  if (m0 + BM <= M && n0 + BN <= N && (N & 7) == 0) {
-    // Interior tile. A lane holds 4 consecutive n of 16 different rows per MFMA tile; storing
-    // that directly makes 32-byte write requests. Instead each wavefront transposes its
-    // sub-tile through LDS (idle now), 64 rows at a time: 8-byte LDS writes in the MFMA
-    // layout, 16-byte LDS reads along rows, 16-byte global stores that cover whole
-    // WTN*2-byte row segments (full 128-byte lines).
-    constexpr int RP = WTN * 2 + 32;            // LDS row pitch in bytes (pad spreads banks)
-    constexpr int kMinBuf = A_BYTES < B_BYTES ? A_BYTES : B_BYTES;
-    constexpr int HM0 = TM < 4 ? TM : 4;        // MFMA tiles (of 16 rows) per pass, halved until
-    constexpr int HM = HM0 * 16 * RP <= kMinBuf ? HM0 : (HM0 / 2) * 16 * RP <= kMinBuf ? HM0 / 2 : 1;  // it fits a buffer
-    constexpr int LPR = WTN * 2 / 16;           // lanes per row on the read side
-    constexpr int RPI = 64 / LPR;               // rows per read instruction
-    static_assert(HM * 16 * RP <= A_BYTES && HM * 16 * RP <= B_BYTES, "epilogue staging: one buffer per wavefront");
-    __syncthreads();  // every wavefront is done reading fragments
-    uint8_t* region = wave == 0 ? a_buf0 : wave == 1 ? a_buf1 : wave == 2 ? b_buf0 : b_buf1;
-    const uint16_t* bias_lane = bias + (has_bias ? n0 + wn + 4 * g : 0);
-    float bv[TN][4];
-    static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
-      constexpr int t = decltype(t_tag)::value;
-      bv[t][0] = bv[t][1] = bv[t][2] = bv[t][3] = 0.f;
-      if (has_bias) {
-        const uint2 braw = *reinterpret_cast<const uint2*>(bias_lane + t * 16);
-        bv[t][0] = unpack1<OUT>(braw.x & 0xFFFFu); bv[t][1] = unpack1<OUT>(braw.x >> 16);
-        bv[t][2] = unpack1<OUT>(braw.y & 0xFFFFu); bv[t][3] = unpack1<OUT>(braw.y >> 16);
-      }
-    });
-    uint8_t* out_base = reinterpret_cast<uint8_t*>(C) + ((size_t)(m0 + wm) * N + n0 + wn) * 2;
-    const int rd_row = lane / LPR, rd_col = (lane % LPR) * 16;
-    static_for<TM / HM>([&](auto p_tag) __attribute__((always_inline)) {
-      constexpr int pass = decltype(p_tag)::value;
-      static_for<HM>([&](auto j_tag) __attribute__((always_inline)) {
-        constexpr int jj = decltype(j_tag)::value;
-        constexpr int j = pass * HM + jj;
-        static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
-          constexpr int t = decltype(t_tag)::value;
-          float o[4];
-#pragma unroll
-          for (int v = 0; v < 4; ++v) o[v] = MX ? acc[t][j][v] + bv[t][v] : acc[t][j][v] * post + bv[t][v];
-          *reinterpret_cast<uint2*>(region + (jj * 16 + r16) * RP + (t * 16 + 4 * g) * 2) =
-              make_uint2(pack2<OUT>(o[0], o[1]), pack2<OUT>(o[2], o[3]));
-        });
-      });
-      // only this wavefront touches its region: LDS operations of one wavefront stay in order
-      static_for<HM * 16 / RPI>([&](auto i_tag) __attribute__((always_inline)) {
-        constexpr int i = decltype(i_tag)::value;
-        const int row = i * RPI + rd_row;  // within the pass
-        const uint4 v = *reinterpret_cast<const uint4*>(region + row * RP + rd_col);
-        *reinterpret_cast<uint4*>(out_base + (size_t)(pass * HM * 16 + row) * N * 2 + rd_col) = v;
-      });
-    });
-    return;
-  }
-  const bool vec_ok = (N & 3) == 0;
-#pragma unroll
-  for (int t = 0; t < TN; ++t) {
-    const int n = n0 + wn + t * 16 + 4 * g;
-    float bv[4] = {0.f, 0.f, 0.f, 0.f};
-    if (has_bias) {
-#pragma unroll
-      for (int v = 0; v < 4; ++v)
-        if (n + v < N) bv[v] = unpack1<OUT>(bias[n + v]);
-    }
-#pragma unroll
-    for (int j = 0; j < TM; ++j) {
-      const int m = m0 + wm + j * 16 + r16;
-      if (m >= M || n >= N) continue;
-      float o[4];
-#pragma unroll
-      for (int v = 0; v < 4; ++v) o[v] = MX ? acc[t][j][v] + bv[v] : acc[t][j][v] * post + bv[v];
-      uint16_t* dst = C + (size_t)m * N + n;
-      if (vec_ok && n + 3 < N) {
-        *reinterpret_cast<uint2*>(dst) = make_uint2(pack2<OUT>(o[0], o[1]), pack2<OUT>(o[2], o[3]));
-      } else {
-#pragma unroll
-        for (int v = 0; v < 4; ++v)
-          if (n + v < N) dst[v] = (uint16_t)(pack2<OUT>(o[v], 0.f) & 0xFFFFu);
-      }
-    }
-  }
+  store_tile<BM, BN, OUT, !MX>(acc, post, nullptr, bias, C, M, N, m0, n0, a_buf0, a_buf1, b_buf0, b_buf1);
 }
 
 struct GemmConfig {

@@ -62,7 +62,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.km_gemm_mx.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_gemm_fp8_tensor.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_wo_gemm_fwd.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
-    lib.km_wo_gemm_dgrad.argtypes = [p, p, p, p, i64, i64, i64, i32, i32, i32, p]
+    lib.km_wo_gemm_dgrad.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_num_configs.argtypes = [i32]
     lib.km_config_desc.argtypes = [i32, i32, c.c_char_p, i32]
     for name in EXPORTS:
@@ -298,8 +298,9 @@ def wo_gemm_dgrad(dy: Tensor, q: Tensor, scale: Tensor, config: int = 0) -> Tens
     m, n = dy.shape
     k = q.shape[1]
     dx = torch.empty(m, k, device=dy.device, dtype=dy.dtype)
+    work = torch.empty(max(n * k, 1), device=dy.device, dtype=torch.uint8)  # codes transposed to [K, N]
     with torch.cuda.device(dy.device):
-        _check(load().km_wo_gemm_dgrad(dy.data_ptr(), q.data_ptr(), scale.data_ptr(), dx.data_ptr(), m, n, k, _QFORMATS[q.dtype], _dtype_code(dy.dtype), config, _stream(dy)))
+        _check(load().km_wo_gemm_dgrad(dy.data_ptr(), q.data_ptr(), scale.data_ptr(), dx.data_ptr(), work.data_ptr(), m, n, k, _QFORMATS[q.dtype], _dtype_code(dy.dtype), config, _stream(dy)))
     return dx
 
 

@@ -1,0 +1,126 @@
+"""HIP weight-only dequant-GEMMs through the C ABI against the fp64 product with the exact
+dequantized weight, next to the oracle's eager result (dequantize, then a 16-bit matmul),
+with the reference's pass rule. Mirrors reference `tests/kernels/quant/test_quant.py`
+(off-tile shapes, int8 and fp8 codes, both 16-bit dtypes, bias on and off, the
+wrong-scale-axis negative control)."""
+
+import pytest
+import torch
+
+from kohakumosstrainer_amd import native
+from oracle import linear
+from oracle.stats import assert_no_regression, rel_l2
+
+pytestmark = pytest.mark.gpu
+SHAPES = ((200, 150, 136), (1, 96, 64), (513, 384, 1000), (300, 256, 512), (1024, 512, 256))
+
+
+def must_fail(check, what=""):
+    try:
+        check()
+    except AssertionError:
+        return
+    raise AssertionError(f"check passed on the broken variant: {what}")
+
+
+def case(m, n, k, fmt, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(n, k, generator=g) * 0.05
+    q, scale = linear.quantize_weight(w, fmt)
+    x = torch.randn(m, k, generator=g).to(dtype)
+    bias = (torch.randn(n, generator=g) * 0.1).to(dtype)
+    dy = torch.randn(m, n, generator=g).to(dtype)
+    return x, q, scale, bias, dy
+
+
+def n_configs():
+    return len(native.configs(native.KERNEL_WO_FWD))
+
+
+@pytest.mark.parametrize("fmt", ("int8", "fp8"))
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+@pytest.mark.parametrize("m,n,k", SHAPES)
+@pytest.mark.parametrize("with_bias", (False, True))
+def test_forward_and_dgrad(fmt, dtype, m, n, k, with_bias):
+    x, q, scale, bias, dy = case(m, n, k, fmt, dtype)
+    b = bias if with_bias else None
+    w64 = linear.wo_exact64(q, scale)
+    truth = x.double() @ w64.T + (b.double() if with_bias else 0)
+    eager = linear.wo_forward(x, q, scale, b)
+    tol = 2e-3 if dtype == torch.bfloat16 else 4e-4
+    for cfg in range(n_configs()):
+        y = native.wo_gemm_fwd(x.cuda(), q.cuda(), scale.cuda(), None if b is None else b.cuda(), cfg)
+        assert y.shape == (m, n) and y.dtype == dtype
+        assert_no_regression(y.cpu(), eager, truth, f"wo fwd {fmt} cfg{cfg} {m}x{n}x{k}")
+        assert rel_l2(y.cpu(), truth) <= tol
+    truth_dx = dy.double() @ w64
+    eager_dx = linear.wo_dgrad(dy, q, scale)
+    for cfg in (0, n_configs() - 1):
+        dx = native.wo_gemm_dgrad(dy.cuda(), q.cuda(), scale.cuda(), cfg)
+        assert dx.shape == (m, k) and dx.dtype == dtype
+        assert_no_regression(dx.cpu(), eager_dx, truth_dx, f"wo dgrad {fmt} cfg{cfg} {m}x{n}x{k}")
+
+
+def test_int8_forward_is_exact_product_for_small_integers():
+    """Integer activations and codes with unit scales: every product and partial sum is an
+    integer below 2^24, so the kernel must reproduce the fp64 product exactly after the one
+    bf16 rounding."""
+    g = torch.Generator().manual_seed(3)
+    m, n, k = 130, 192, 320
+    x = torch.randint(-4, 5, (m, k), generator=g).to(torch.bfloat16)
+    q = torch.randint(-127, 128, (n, k), generator=g).to(torch.int8)
+    scale = torch.ones(n)
+    y = native.wo_gemm_fwd(x.cuda(), q.cuda(), scale.cuda(), None, 0).cpu()
+    want = (x.double() @ q.double().T).to(torch.bfloat16)
+    assert torch.equal(y, want)
+
+
+@pytest.mark.parametrize("fmt", ("int8", "fp8"))
+def test_error_check_rejects_wrong_scale_axis(fmt):
+    m, n, k = 64, 96, 96
+    x, q, scale, _, _ = case(m, n, k, fmt, torch.bfloat16)
+    eager = linear.wo_forward(x, q, scale, None)
+    truth = x.double() @ linear.wo_exact64(q, scale).T
+    good = native.wo_gemm_fwd(x.cuda(), q.cuda(), scale.cuda(), None, 0).cpu()
+    assert_no_regression(good, eager, truth, "good")
+    scale_in = scale[torch.arange(k) % n]
+    broken = (x.float() @ (q.float() * scale_in[None, :]).T).to(torch.bfloat16)
+    must_fail(lambda: assert_no_regression(broken, eager, truth, "broken"), "scale along the input axis")
+    rolled = native.wo_gemm_fwd(x.cuda(), q.cuda(), (scale * torch.where(torch.arange(n) % 2 == 0, 1.0, 64.0)).roll(1).cuda(), None, 0).cpu()
+    must_fail(lambda: assert_no_regression(rolled, eager, truth, "rolled"), "scales on the wrong rows")
+
+
+def test_int8_weight_only_frozen_base_shape():
+    """x bf16 [4096, 3072], W int8 [3072, 3072] uniform in [-127, 127], scale |N(0,0.02)|/127 + 1e-6,
+    fp32 bias ~N(0,0.01): a 256-row slice against the fp64 product, and the whole output
+    against the slice-wise property that rows are independent (permutation equivariance)."""
+    g = torch.Generator().manual_seed(0)
+    m, k, n = 4096, 3072, 3072
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    q = torch.randint(-127, 128, (n, k), generator=g).to(torch.int8)
+    scale = torch.randn(n, generator=g).abs() * 0.02 / 127 + 1e-6
+    bias = torch.randn(n, generator=g) * 0.01
+    xg, qg, sg, bg = x.cuda(), q.cuda(), scale.cuda(), bias.to(torch.bfloat16).cuda()
+    y = native.wo_gemm_fwd(xg, qg, sg, bg, 0)
+    rows = torch.arange(1000, 1256)
+    truth = x[rows].double() @ linear.wo_exact64(q, scale).T + bias.to(torch.bfloat16).double()
+    eager = linear.wo_forward(x[rows], q, scale, bias)
+    assert_no_regression(y[rows].cpu(), eager, truth, "int8 frozen base")
+    assert rel_l2(y[rows].cpu(), truth) <= 2e-3
+    perm = torch.randperm(m, generator=g).cuda()
+    assert torch.equal(native.wo_gemm_fwd(xg[perm].contiguous(), qg, sg, bg, 0), y[perm])
+
+
+def test_argument_errors():
+    x = torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda")
+    q = torch.zeros(16, 64, dtype=torch.int8, device="cuda")
+    s = torch.ones(16, device="cuda")
+    with pytest.raises(ValueError):
+        native.wo_gemm_fwd(x, q.float(), s, None)
+    with pytest.raises(ValueError):
+        native.wo_gemm_fwd(x, q[:, :32], s, None)
+    with pytest.raises(ValueError):
+        native.wo_gemm_fwd(x, q, s[:3], None)
+    with pytest.raises(native.KernelError):
+        native.wo_gemm_fwd(x, q, s, None, 99)
+    assert native.wo_gemm_fwd(x[:0], q, s, None).shape == (0, 16)
