@@ -81,6 +81,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", type=int, default=0, help="GEMM tile configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate", action="store_true", help="also run 5 plain device copies of the activation tensor (a kernel of known HBM traffic, to scale profiler byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path needs no second GPU); use --gpus 1")
@@ -98,6 +99,10 @@ def main():
         xq, _, xsp = native.quant_mx(x, natural=False, packed=True)
         return native.gemm_mx(xq, xsp, wq, wsp, bias, torch.bfloat16, args.config, packed=True)
 
+    if args.calibrate:
+        sink = torch.empty_like(x)
+        for _ in range(5):
+            sink.copy_(x)  # reads and writes M*K*2 bytes each
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

@@ -1,0 +1,107 @@
+"""HIP backend of `fp8_linear` on gfx950: the GEMM paths of the form c = Q(a) B^T (forward:
+a = x, B = W; fp8 input gradient: a = dy, B = W^T, the dgrad copy), one tile configuration per
+problem picked by the tuner and bound once settled. Each path includes its activation
+quantizer. Host-side counterpart of reference `backends/triton/fp8/linear.py` (candidates
+:88-118, runner :162-196, `_select` :254-286, launchers :289-301, registration :309-320).
+
+Recipes served on the GPU: `mx` (block-scaled MFMA; the activation quantizer writes the
+MFMA-packed scales directly, the weight's packed copy comes in `aux` or is packed per call)
+and `tensor` (plain fp8 MFMA, scalar scales on the accumulator). `row` and `block` are not
+built yet and are refused by the support check. The 16-bit input gradient of a base stored
+without a dgrad copy is `dy @ dequantize(W)`: an elementwise dequantize and a plain library
+GEMM, as in the reference's `w16` path.
+"""
+
+import torch
+
+from kohakumosstrainer_amd import native
+from kohakumosstrainer_amd.kernels import registry, tuning
+from kohakumosstrainer_amd.kernels.constraints import requires
+from kohakumosstrainer_amd.kernels.errors import BackendUnavailable
+from kohakumosstrainer_amd.kernels.fp8.formats import dequantize, packed_numel
+from kohakumosstrainer_amd.kernels.fp8.op import make_fp8_linear, make_fp8_linear_infer, register_launchers
+from kohakumosstrainer_amd.kernels.fp8.train import make_fp8_linear_train
+from kohakumosstrainer_amd.kernels.tuning import pow2
+
+GPU_RECIPES = ("mx", "tensor")
+ALIGN_K = 128
+_RESOLVED: dict[tuple, dict] = {}
+tuning.on_reset(_RESOLVED.clear)
+
+
+def candidates(recipe: str, m: int) -> list[dict]:
+    """Tile configurations of the fp8 GEMM for M rows, the planner's first pick first: large
+    tiles for large M (fewest bytes fetched per flop), smaller ones when M is short or the
+    grid would not fill 256 CUs."""
+    cfgs = [{"gemm": "hip", **c} for c in native.configs(native.KERNEL_GEMM_MX if recipe == "mx" else native.KERNEL_GEMM_FP8)]
+    limit = max(pow2(m, 16), min(c["bm"] for c in cfgs))
+    fits = [c for c in cfgs if c["bm"] <= limit] or cfgs
+    return sorted(fits, key=lambda c: -(c["bm"] * c["bn"]) if m >= 1024 else c["bm"])
+
+
+def _table_key(kind, m, n, k, a, recipe, bias) -> str:
+    return f"{kind}_m{pow2(m, 16)}_n{n}_k{k}_{a.dtype}_{recipe}_{'x' if bias is None else 'b'}"
+
+
+def _check_shapes(kind, a, bq, recipe):
+    if recipe not in GPU_RECIPES:
+        raise BackendUnavailable(f"fp8_{kind}", {"hip": f"recipe {recipe!r} is not built for gfx950 yet"}, persist=False)
+    if a.shape[1] % ALIGN_K or bq.shape[1] != a.shape[1]:
+        raise ValueError(f"fp8_{kind}: contraction length {a.shape[1]} (weight {tuple(bq.shape)}) must match and be a multiple of {ALIGN_K}")
+
+
+def _run(cfg, recipe, a, bq, bs, baux, bias):
+    """(a16 [M, K], bq [N, K], bs, baux, bias) -> Q(a) bq^T in a's dtype with tile config `cfg`."""
+    if recipe == "mx":
+        aq, _, a_packed = native.quant_mx(a, natural=False, packed=True)
+        if baux is None or baux.numel() != packed_numel(bq.shape[0], bq.shape[1]) or baux.dtype != torch.uint8:
+            baux = native.pack_scales(bs)
+        return native.gemm_mx(aq, a_packed, bq, baux, bias, a.dtype, cfg["id"], packed=True)
+    aq, sa = native.quant_tensor(a)
+    return native.gemm_fp8_tensor(aq, sa, bq, bs.reshape(1).float(), bias, a.dtype, cfg["id"])
+
+
+def _select(kind, a, bq, bs, baux, bias, recipe, in_backward):
+    m, k = a.shape
+    n = bq.shape[0]
+    key = (kind, a.device.index, pow2(m, 16), n, k, a.dtype, recipe, bias is None)
+    cfg = _RESOLVED.get(key)
+    if cfg is not None:
+        return cfg
+    table_key = _table_key(kind, m, n, k, a, recipe, bias)
+    cfg = tuning.select(
+        f"fp8_{kind}",
+        a.device,
+        table_key,
+        lambda: candidates(recipe, m),
+        lambda c: lambda: _run(c, recipe, a, bq, bs, baux, bias),
+        shortlist=8,
+        in_backward=in_backward,
+    )
+    if tuning.decided(f"fp8_{kind}", a.device, table_key):
+        _RESOLVED[key] = cfg
+    return cfg
+
+
+def fwd(x, q, scale, aux, bias, recipe):
+    _check_shapes("fwd", x, q, recipe)
+    cfg = _select("fwd", x, q, scale, aux, bias, recipe, False)
+    return _run(cfg, recipe, x, q, scale, aux, bias)
+
+
+def dgrad(dy, q, scale, q_t, scale_t, aux_t, recipe):
+    if q_t is None:
+        return dy @ dequantize(q, scale, recipe, dy.dtype)
+    _check_shapes("dgrad", dy, q_t, recipe)
+    cfg = _select("dgrad", dy, q_t, scale_t, aux_t, None, recipe, True)
+    return _run(cfg, recipe, dy, q_t, scale_t, aux_t, None)
+
+
+def _gpu_recipe(query):
+    recipe = query.get("recipe", "row")
+    return None if recipe in GPU_RECIPES else f"fp8 recipe {recipe!r} is not built for gfx950 (have {GPU_RECIPES})"
+
+
+register_launchers("hip", fwd, dgrad)
+for _op, _make in (("fp8_linear", make_fp8_linear), ("fp8_linear_infer", make_fp8_linear_infer), ("fp8_linear_train", make_fp8_linear_train)):
+    registry.register(_op, "hip", _make("hip"), supports=requires(kinds=("hip",), archs=("gfx950",), extra=_gpu_recipe))
