@@ -25,7 +25,11 @@ FP8_PEAK_TFLOPS = 5000.0  # MI355X dense fp8 / MXFP8 MFMA
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 GEMM_FLOP = 2 * M * N * K
 QUANT_BYTES = M * K * 2 + M * K + M * K // 32  # bf16 read + codes + scale bytes, per direction
-CPU_SAMPLE_ROWS = 512
+CPU_SAMPLE_ROWS = 16384  # the whole workload: this host's cores finish it in seconds
+# HBM-side bytes of one GEMM launch from the profiler's FETCH_SIZE / WRITE_SIZE counters
+# (profiles/gemm_fp8_kernel_M16384_K3072_N9216_pmc.txt), each scaled by what the same counter
+# reads for a plain 100 663 296-byte device copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0).
+GEMM_TRAFFIC_BYTES = 1_003_000_000
 
 
 def synthetic(device):
@@ -59,7 +63,7 @@ def cpu_baseline(x, wq, ws, bias):
     xs = x[:CPU_SAMPLE_ROWS].cpu()
     wq_c, ws_c, b_c = wq.cpu(), ws.cpu(), bias.cpu()
     best = float("inf")
-    for _ in range(3):
+    for _ in range(5):
         t = time.perf_counter()
         linear.fp8_forward(xs, wq_c, ws_c, None, b_c, "mx")
         best = min(best, time.perf_counter() - t)
@@ -70,8 +74,53 @@ def cpu_baseline(x, wq, ws, bias):
         "cores": torch.get_num_threads(),
         "host_cpus": os.cpu_count(),
         "kind": "port",
-        "sample": f"first {CPU_SAMPLE_ROWS} of {M} rows, full W [{N},{K}]: quantize + dequantize + bf16 linear, best of 3 ({best:.2f} s)",
+        "sample": f"{CPU_SAMPLE_ROWS} of {M} rows, full W [{N},{K}]: quantize x, dequantize x and W, bf16 linear + bias (torch CPU), best of 5 ({best:.2f} s each)",
     }
+
+
+def other_configs(dev, reps):
+    """Device time of the other kernels of the path at their BASELINE shapes (event-timed,
+    back to back): weight-only int8 / e4m3 GEMMs and the frozen-base MXFP8 forward + input
+    gradient of the adapter-training shape."""
+    from kohakumosstrainer_amd import native
+
+    g = torch.Generator(device="cpu").manual_seed(0)
+    out = {}
+    for name, (m, k, n), fmt in (("wo_int8_M4096_K3072_N3072", (4096, 3072, 3072), "int8"), ("wo_e4m3_M8192_K3072_N12288", (8192, 3072, 12288), "fp8")):
+        x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(dev)
+        if fmt == "int8":
+            q = torch.randint(-127, 128, (n, k), generator=g).to(torch.int8).to(dev)
+        else:
+            q = (torch.randn(n, k, generator=g) * 100).to(torch.float8_e4m3fn).to(dev)
+        scale = (torch.rand(n, generator=g) * 1e-3 + 1e-6).to(dev)
+        bias = torch.zeros(n, dtype=torch.bfloat16, device=dev)
+        dy = torch.randn(m, n, generator=g).to(torch.bfloat16).to(dev)
+        native.wo_gemm_fwd(x, q, scale, bias, 0)
+        native.wo_gemm_dgrad(dy, q, scale, 0)
+        f = event_ms(lambda: native.wo_gemm_fwd(x, q, scale, bias, 0), reps)
+        d = event_ms(lambda: native.wo_gemm_dgrad(dy, q, scale, 0), reps)
+        flop = 2 * m * n * k
+        out[name] = {"fwd_ms": f, "fwd_TFLOPs": flop / f / 1e9, "dgrad_ms": d, "dgrad_TFLOPs": flop / d / 1e9, "peak_TFLOPs": 2500.0}
+    m, k, n = 2048, 4096, 12288
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(n, k, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+    dy = (torch.randn(m, n, generator=g) * 0.01).to(torch.bfloat16).to(dev)
+    wq, _, wsp = native.quant_mx(w, natural=False, packed=True)
+    wtq, _, wtsp = native.quant_mx(w.t(), natural=False, packed=True)
+
+    def fwd():
+        xq, _, xsp = native.quant_mx(x, natural=False, packed=True)
+        return native.gemm_mx(xq, xsp, wq, wsp, None, torch.bfloat16, 0, packed=True)
+
+    def dgrad():
+        gq, _, gsp = native.quant_mx(dy, natural=False, packed=True)
+        return native.gemm_mx(gq, gsp, wtq, wtsp, None, torch.bfloat16, 0, packed=True)
+
+    fwd(), dgrad()
+    f, d = event_ms(fwd, reps), event_ms(dgrad, reps)
+    flop = 2 * m * n * k
+    out["mx_frozen_base_M2048_K4096_N12288"] = {"fwd_ms": f, "fwd_TFLOPs": flop / f / 1e9, "dgrad_ms": d, "dgrad_TFLOPs": flop / d / 1e9, "peak_TFLOPs": FP8_PEAK_TFLOPS, "note": "quantizer + GEMM per call"}
+    return out
 
 
 def main():
@@ -113,9 +162,16 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
 
-    # per-kernel device time, measured live with events
-    xq, _, xsp = native.quant_mx(x, natural=False, packed=True)
-    gemm_ms = event_ms(lambda: native.gemm_mx(xq, xsp, wq, wsp, bias, torch.bfloat16, args.config, packed=True), max(args.steps, 10))
+    # per-kernel device time, measured live with events: the GEMM inside the same step sequence
+    # (its launch follows the quantizer's, as in the timed region), the quantizers back to back
+    marks = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for before, after in marks:
+        xq, _, xsp = native.quant_mx(x, natural=False, packed=True)
+        before.record()
+        native.gemm_mx(xq, xsp, wq, wsp, bias, torch.bfloat16, args.config, packed=True)
+        after.record()
+    torch.cuda.synchronize()
+    gemm_ms = sum(b.elapsed_time(a) for b, a in marks) / len(marks)
     rows_ms = event_ms(lambda: native.quant_mx(x), max(args.steps, 10))
     fused_rows_ms = event_ms(lambda: native.quant_mx(x, natural=False, packed=True), max(args.steps, 10))
     xt = x.t()
@@ -146,7 +202,8 @@ def main():
             "peak": FP8_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / FP8_PEAK_TFLOPS,
-            "traffic": None,
+            "traffic": GEMM_TRAFFIC_BYTES,
+            "algorithmic_flop": GEMM_FLOP,
             "ms": gemm_ms,
         },
         "quantizer": {
@@ -163,6 +220,7 @@ def main():
             "unit": "GB/s",
         },
     }
+    line["other_configs"] = other_configs(dev, max(args.steps // 2, 5))
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(x, wq, ws, bias)
     print(json.dumps(line))

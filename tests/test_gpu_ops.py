@@ -58,9 +58,9 @@ def exact_product(a, q, scale, bias, recipe):
     return y if bias is None else y + bias.double()
 
 
-def check(got, eager, exact, dtype, what):
+def check(got, eager, exact, dtype, what, slack=1.0):
     rel = oracle_stats.rel_l2(got.cpu(), exact)
-    assert rel <= REL_L2[dtype], (what, rel)
+    assert rel <= REL_L2[dtype] * slack, (what, rel)
     oracle_stats.assert_no_regression(got.cpu(), eager, exact, name=what)
 
 
@@ -139,7 +139,9 @@ def test_quant_linear_op(dtype, fmt):
     w64 = oracle_linear.wo_exact64(q, scale)
     exact_y, exact_dx = x.double() @ w64.T + bias.double(), dy.double() @ w64
     check(y.detach(), oracle_linear.wo_forward(x, q, scale, bias), exact_y, dtype, f"wo fwd {fmt}")
-    check(xd.grad, oracle_linear.wo_dgrad(dy, q, scale), exact_dx, dtype, f"wo dgrad {fmt}")
+    # the per-row scale lies on the contraction axis of the input gradient, so it is folded into
+    # a 16-bit operand (one extra rounding, as in the eager launcher): twice the forward bound
+    check(xd.grad, oracle_linear.wo_dgrad(dy, q, scale), exact_dx, dtype, f"wo dgrad {fmt}", slack=2.0)
 
 
 def test_shortlist_is_timed_once_and_stored(tmp_path, monkeypatch):
@@ -150,11 +152,11 @@ def test_shortlist_is_timed_once_and_stored(tmp_path, monkeypatch):
     x, w, bias, dy, base = problem(512, 512, 512, torch.bfloat16, "mx")
     op = registry.resolve("fp8_linear", DEV, torch.bfloat16, recipe="mx")
     args = parts(base, DEV)
-    before = tuning.TIMED.get("fp8_linear", 0)
+    before = tuning.TIMED.get("fp8_fwd", 0)
     a = op(x.to(DEV), *args, bias.to(DEV), "mx")
     b = op(x.to(DEV), *args, bias.to(DEV), "mx")
-    assert tuning.TIMED.get("fp8_linear", 0) == before + 1 and torch.equal(a, b)
-    rows = [p for p in tmp_path.rglob("fp8_linear.json")]
+    assert tuning.TIMED.get("fp8_fwd", 0) == before + 1 and torch.equal(a, b)
+    rows = [p for p in tmp_path.rglob("fp8_fwd.json")]
     assert len(rows) == 1 and "fwd_m512_n512_k512" in rows[0].read_text()
     tuning._tables.clear()
 

@@ -166,3 +166,20 @@ def test_tensor_recipe_all_zero_and_weight_like():
     q, s = native.quant_tensor(w.cuda())
     rq, rs = formats.quantize(w, "tensor")
     assert torch.equal(s.cpu(), rs) and torch.equal(u8(q).cpu(), u8(rq))
+
+
+def test_mx_committed_vectors_rows_and_cols():
+    """The committed known-answer bytes (definition-level, independent of the oracle): the
+    row-wise kernel on the vectors as they are, the column-wise kernel on their transpose."""
+    from pathlib import Path
+
+    import numpy as np
+
+    d = np.load(Path(__file__).parent / "golden" / "mx_vectors.npz")
+    x = torch.from_numpy(d["x_bits"].astype(np.int32)).to(torch.uint16).view(torch.bfloat16)
+    want_q, want_s = torch.from_numpy(d["codes"]), torch.from_numpy(d["scales"])
+    q, s = native.quant_mx(x.cuda())
+    assert torch.equal(u8(q).cpu(), want_q) and torch.equal(s.cpu(), want_s)
+    xt = x.t().contiguous().cuda()  # [128, R]: quantizing xt.t() runs the transposing kernel
+    q2, s2 = native.quant_mx(xt.t())
+    assert torch.equal(u8(q2).cpu(), want_q) and torch.equal(s2.cpu(), want_s)

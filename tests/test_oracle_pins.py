@@ -379,3 +379,36 @@ def test_linears_against_fp64_products():
     out = linear.lora_bypass(y, x, down, up, 1.0)
     closed = y.double() + x.double() @ (up.double() @ down.double()).T
     assert rel_l2(out, closed) < 1e-2
+
+
+# ---- committed known-answer vectors ----------------------------------------------------
+
+
+def golden():
+    from pathlib import Path
+
+    return np.load(Path(__file__).parent / "golden" / "mx_vectors.npz")
+
+
+def test_oracle_reproduces_committed_mx_vectors():
+    """Both restatements (torch and C) against the committed bytes, which were produced by
+    the definition-level routines of `tests/_independent.py` (`tests/golden/make_vectors.py`)."""
+    d = golden()
+    bits = torch.from_numpy(d["x_bits"].astype(np.int32)).to(torch.uint16)
+    x = bits.view(torch.bfloat16)
+    q, s = formats.quantize(x, "mx", "act")
+    assert np.array_equal(u8(q), d["codes"]) and np.array_equal(s.numpy(), d["scales"])
+    lib = oracle_build.load()
+    rows, k = d["x_bits"].shape
+    cq = np.zeros((rows, k), dtype=np.uint8)
+    cs = np.zeros((rows, k // 32), dtype=np.uint8)
+    xb = np.ascontiguousarray(d["x_bits"])
+    lib.oracle_mx_quantize_bf16(xb.ctypes.data, rows, k, k, 1, cq.ctypes.data, cs.ctypes.data)
+    assert np.array_equal(cq, d["codes"]) and np.array_equal(cs, d["scales"])
+    must_fail(lambda: np.testing.assert_array_equal(u8(formats.quantize(x * 2, "mx", "act")[1]), d["scales"]), "scaled input")
+
+
+def test_weight_quantizer_reproduces_committed_int8_vectors():
+    d = golden()
+    q, s = linear.quantize_weight(torch.from_numpy(d["w_int8_in"]), "int8")
+    assert np.array_equal(q.numpy(), d["w_int8_q"]) and np.array_equal(s.numpy(), d["w_int8_scale"])
