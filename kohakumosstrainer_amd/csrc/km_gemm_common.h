@@ -82,6 +82,40 @@ constexpr int kWaitVm0 = 0x0F70;         // vmcnt(0)
 constexpr int kWaitLgkm0 = 0xC07F;       // lgkmcnt(0)
 constexpr int wait_vm_lgkm0(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070; }  // vmcnt(n) lgkmcnt(0)
 
+// ---- vector-memory reads the compiler does not see ------------------------------------------
+// The compiler cannot tell which LDS buffer a direct-to-LDS load fills and answers every later
+// LDS read with s_waitcnt vmcnt(0), which drains the prefetches that are meant to stay in
+// flight across a K step. Issued from inline asm, the loads are invisible to that bookkeeping:
+// the only vmcnt waits left are the explicit ones of the kernel, and every result is used after
+// one of them (a "memory" clobber keeps LDS reads from moving across). The hazard recognizer
+// does not look into inline asm either: an SGPR written by a VALU instruction (v_readfirstlane,
+// the reload of a spilled SGPR) must not be read by a vector-memory instruction within 5 wait
+// states, and m0 not within 1, hence the s_nop in front of each.
+__device__ __forceinline__ uint32_t lds_offset(const void* p) {
+  return (uint32_t)reinterpret_cast<uintptr_t>((lds_ptr_t)const_cast<void*>(p));
+}
+// raw buffer descriptor (stride 0, range check on the per-lane offset) from uniform values
+__device__ __forceinline__ v4i raw_rsrc(const void* base, uint32_t bytes) {
+  const uint64_t b = (uint64_t)reinterpret_cast<uintptr_t>(base);
+  return v4i{__builtin_amdgcn_readfirstlane((int)(uint32_t)b), __builtin_amdgcn_readfirstlane((int)((uint32_t)(b >> 32) & 0xFFFFu)),
+             __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
+}
+// each lane fetches 16 bytes at voffset (+ soffset); they land at lds_addr + 16 * lane
+__device__ __forceinline__ void hidden_dma_b128(const v4i& rsrc, uint32_t lds_addr, int voffset, int soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               ::"s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+}
+__device__ __forceinline__ uint64_t hidden_load_b64(const v4i& rsrc, int voffset, int soffset) {
+  uint64_t v;
+  asm volatile("s_nop 4\n\tbuffer_load_dwordx2 %0, %1, %2, %3 offen" : "=v"(v) : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+  return v;
+}
+__device__ __forceinline__ uint32_t hidden_load_b32(const v4i& rsrc, int voffset, int soffset) {
+  uint32_t v;
+  asm volatile("s_nop 4\n\tbuffer_load_dword %0, %1, %2, %3 offen" : "=v"(v) : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+  return v;
+}
+
 // Epilogue of a 2 x 2 wavefront grid over a BM x BN tile of 16x16 MFMA tiles whose rows are
 // output columns: lane (r16 = lane%16, g = lane/16) of tile (t, j) holds
 // C[m0+wm+j*16+r16][n0+wn+t*16+4g .. +3]. Computes acc * post * col_scale[n] + bias[n] in fp32,

@@ -104,10 +104,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
 
   // buffer descriptors start at this tile's first row; their range check (on the per-lane
   // offset) turns rows past the end into zeros
-  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint8_t*>(A) + (size_t)m0 * K, 0, (int)min((int64_t)(M - m0) * K, (int64_t)0x7FFFFFFF), 0x00020000);
-  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint8_t*>(B) + (size_t)n0 * K, 0, (int)min((int64_t)(N - n0) * K, (int64_t)0x7FFFFFFF), 0x00020000);
+  const v4i a_rsrc = raw_rsrc(A + (size_t)m0 * K, (uint32_t)min((int64_t)(M - m0) * K, (int64_t)0x7FFFFFFF));
+  const v4i b_rsrc = raw_rsrc(B + (size_t)n0 * K, (uint32_t)min((int64_t)(N - n0) * K, (int64_t)0x7FFFFFFF));
   // staging map of a pass: 8 lanes per row; 16 lanes cover rows r and r+8 (one LDS line)
   const int w = tid >> 3;
   const int srow = ((w >> 4) << 4) + ((w & 1) << 3) + ((w >> 1) & 7);  // 0 .. 31
@@ -116,15 +114,15 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
   const int pass_stride = 32 * K;
 
   // scales: MFMA rows come from B (n), MFMA columns from A (m)
-  __amdgpu_buffer_rsrc_t ws_rsrc, xs_rsrc;
+  v4i ws_rsrc, xs_rsrc;
   int ws_off[SCALE_KM ? 1 : TN], xs_off[SCALE_KM ? 1 : TM];
   int ws_step = 0, xs_step = 0, ws_base = 0, xs_base = 0, ws_sel = 0, xs_sel = 0;
   if constexpr (MX) {
     if constexpr (SCALE_KM) {
       // packed: byte offset ((ks*RB + r/128)*16 + r%16)*32 + 8*block + (r%128)/16
       const int rbn = (N + 127) >> 7, rbm = (M + 127) >> 7;
-      ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(Bs), 0, (int)min((int64_t)nk * rbn * 512, (int64_t)0x7FFFFFFF), 0x00020000);
-      xs_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(As), 0, (int)min((int64_t)nk * rbm * 512, (int64_t)0x7FFFFFFF), 0x00020000);
+      ws_rsrc = raw_rsrc(Bs, (uint32_t)min((int64_t)nk * rbn * 512, (int64_t)0x7FFFFFFF));
+      xs_rsrc = raw_rsrc(As, (uint32_t)min((int64_t)nk * rbm * 512, (int64_t)0x7FFFFFFF));
       ws_off[0] = r16 * 32 + g * 8;
       xs_off[0] = ws_off[0];
       ws_base = min((n0 + wn) >> 7, rbn - 1) * 512;  // waves wholly past the edge read valid bytes
@@ -135,10 +133,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
       xs_sel = (((m0 + wm) & 127) >> 4) * 8;
     } else {
       // natural [rows, K/32]; row indices are clamped to the last valid row
-      ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(Bs) + (size_t)n0 * kb, 0,
-                                                  (int)min((int64_t)(N - n0) * kb, (int64_t)0x7FFFFFFF), 0x00020000);
-      xs_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(As) + (size_t)m0 * kb, 0,
-                                                  (int)min((int64_t)(M - m0) * kb, (int64_t)0x7FFFFFFF), 0x00020000);
+      ws_rsrc = raw_rsrc(Bs + (size_t)n0 * kb, (uint32_t)min((int64_t)(N - n0) * kb, (int64_t)0x7FFFFFFF));
+      xs_rsrc = raw_rsrc(As + (size_t)m0 * kb, (uint32_t)min((int64_t)(M - m0) * kb, (int64_t)0x7FFFFFFF));
       ws_step = 4;
       xs_step = 4;
 #pragma unroll
@@ -165,15 +161,14 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
   // (the inline-asm MFMAs are opaque to the compiler's hazard handling).
   int wscale[2][WS], xscale[2][XS];
   uint32_t wraw[WS], xraw[XS];
+  uint64_t wraw64 = 0, xraw64 = 0;  // packed layout: the 8 scale bytes of a lane
 
   // one 4 KiB pass (32 rows) of a slab: each wavefront moves 1 KiB with one instruction
   auto dma_a_pass = [&](uint8_t* buf, int koff, int i) __attribute__((always_inline)) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(buf + i * 4096 + wave * 1024), 16,
-                                             ld_voff + i * pass_stride, koff, 0, 0);
+    hidden_dma_b128(a_rsrc, lds_offset(buf) + i * 4096 + wave * 1024, ld_voff + i * pass_stride, koff);
   };
   auto dma_b_pass = [&](uint8_t* buf, int koff, int i) __attribute__((always_inline)) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr_t)(buf + i * 4096 + wave * 1024), 16,
-                                             ld_voff + i * pass_stride, koff, 0, 0);
+    hidden_dma_b128(b_rsrc, lds_offset(buf) + i * 4096 + wave * 1024, ld_voff + i * pass_stride, koff);
   };
   auto dma_a = [&](uint8_t* buf, int ks) __attribute__((always_inline)) {
     const int koff = __builtin_amdgcn_readfirstlane(ks * kStepBytes);
@@ -190,17 +185,15 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
       const int wso = __builtin_amdgcn_readfirstlane(ks * ws_step + ws_base);
       const int xso = __builtin_amdgcn_readfirstlane(ks * xs_step + xs_base);
       if constexpr (SCALE_KM) {
-        const uint2 wv = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(ws_rsrc, ws_off[0], wso, 0));
-        const uint2 xv = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(xs_rsrc, xs_off[0], xso, 0));
-        wraw[0] = wv.x; wraw[1] = wv.y;
-        xraw[0] = xv.x; xraw[1] = xv.y;
+        wraw64 = hidden_load_b64(ws_rsrc, ws_off[0], wso);
+        xraw64 = hidden_load_b64(xs_rsrc, xs_off[0], xso);
       } else {
 #pragma unroll
         for (int t = 0; t < TN; ++t)
-          wraw[t] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ws_rsrc, ws_off[t], wso, 0);
+          wraw[t] = hidden_load_b32(ws_rsrc, ws_off[t], wso);
 #pragma unroll
         for (int t = 0; t < TM; ++t)
-          xraw[t] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(xs_rsrc, xs_off[t], xso, 0);
+          xraw[t] = hidden_load_b32(xs_rsrc, xs_off[t], xso);
       }
     }
   };
@@ -214,8 +207,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
 #pragma unroll
       for (int t = 0; t < XS; ++t) xscale[P][t] = (int)(0x7F7F7F7Fu & live);
     } else if constexpr (SCALE_KM) {
-      const uint64_t wv = (((uint64_t)wraw[1] << 32) | wraw[0]) >> ws_sel;
-      const uint64_t xv = (((uint64_t)xraw[1] << 32) | xraw[0]) >> xs_sel;
+      const uint64_t wv = wraw64 >> ws_sel;
+      const uint64_t xv = xraw64 >> xs_sel;
       wscale[P][0] = (int)((uint32_t)wv & live); wscale[P][1] = (int)((uint32_t)(wv >> 32) & live);
       xscale[P][0] = (int)((uint32_t)xv & live); xscale[P][1] = (int)((uint32_t)(xv >> 32) & live);
     } else {
