@@ -62,11 +62,12 @@ def cpu_baseline(x, wq, ws, bias):
 
     xs = x[:CPU_SAMPLE_ROWS].cpu()
     wq_c, ws_c, b_c = wq.cpu(), ws.cpu(), bias.cpu()
-    best = float("inf")
-    for _ in range(5):
+    best, total, reps = float("inf"), 0.0, 0
+    while total < 12.0 and reps < 200:  # about 12 s of CPU work
         t = time.perf_counter()
         linear.fp8_forward(xs, wq_c, ws_c, None, b_c, "mx")
-        best = min(best, time.perf_counter() - t)
+        dt = time.perf_counter() - t
+        best, total, reps = min(best, dt), total + dt, reps + 1
     flop = 2 * CPU_SAMPLE_ROWS * N * K
     return {
         "value": flop / best / 1e12,
@@ -74,7 +75,7 @@ def cpu_baseline(x, wq, ws, bias):
         "cores": torch.get_num_threads(),
         "host_cpus": os.cpu_count(),
         "kind": "port",
-        "sample": f"{CPU_SAMPLE_ROWS} of {M} rows, full W [{N},{K}]: quantize x, dequantize x and W, bf16 linear + bias (torch CPU), best of 5 ({best:.2f} s each)",
+        "sample": f"{CPU_SAMPLE_ROWS} of {M} rows, full W [{N},{K}]: quantize x, dequantize x and W, bf16 linear + bias (torch CPU), best of {reps} passes ({best:.2f} s each, {total:.0f} s in all)",
     }
 
 
@@ -127,8 +128,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=0, help="GEMM tile configuration")
+    ap.add_argument("--warmup", type=int, default=200, help="untimed steps first (about 0.1 s: the card needs that long to reach its sustained clocks)")
+    ap.add_argument("--config", type=int, default=-1, help="GEMM tile configuration; -1 times every configuration once, as the tuning table does, and takes the fastest")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calibrate", action="store_true", help="also run 5 plain device copies of the activation tensor (a kernel of known HBM traffic, to scale profiler byte counters)")
     args = ap.parse_args()
@@ -144,9 +145,20 @@ def main():
     # weights are quantized once, outside the step; the GEMM reads the MFMA-packed scale copy
     wq, ws, wsp = native.quant_mx(w, packed=True)
 
+    xq0, _, xsp0 = native.quant_mx(x, natural=False, packed=True)
+    config, tried = args.config, {}
+    if config < 0:
+        for _ in range(100):  # reach sustained clocks before comparing
+            native.gemm_mx(xq0, xsp0, wq, wsp, bias, torch.bfloat16, 0, packed=True)
+        for cfg in native.configs(native.KERNEL_GEMM_MX):
+            run = lambda c=cfg["id"]: native.gemm_mx(xq0, xsp0, wq, wsp, bias, torch.bfloat16, c, packed=True)
+            event_ms(run, 5)
+            tried[cfg["id"]] = event_ms(run, 20)
+        config = min(tried, key=tried.get)
+
     def step():
         xq, _, xsp = native.quant_mx(x, natural=False, packed=True)
-        return native.gemm_mx(xq, xsp, wq, wsp, bias, torch.bfloat16, args.config, packed=True)
+        return native.gemm_mx(xq, xsp, wq, wsp, bias, torch.bfloat16, config, packed=True)
 
     if args.calibrate:
         sink = torch.empty_like(x)
@@ -168,7 +180,7 @@ def main():
     for before, after in marks:
         xq, _, xsp = native.quant_mx(x, natural=False, packed=True)
         before.record()
-        native.gemm_mx(xq, xsp, wq, wsp, bias, torch.bfloat16, args.config, packed=True)
+        native.gemm_mx(xq, xsp, wq, wsp, bias, torch.bfloat16, config, packed=True)
         after.record()
     torch.cuda.synchronize()
     gemm_ms = sum(b.elapsed_time(a) for b, a in marks) / len(marks)
@@ -193,7 +205,8 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": f"MXFP8 fused-QKV linear forward M={M} K={K} N={N}: per-call activation quantizer + block-scaled GEMM + bias, bf16 out (BASELINE configs[3]); quantizer alone on bf16 [{M},{K}] row- and column-wise (configs[2])",
-            "gemm_tile_config": args.config,
+            "gemm_tile_config": config,
+            "gemm_tile_configs_ms": tried,
         },
         "roofline": {
             "kernel": "gemm_fp8_kernel (MX)",

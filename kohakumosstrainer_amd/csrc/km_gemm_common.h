@@ -187,7 +187,9 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
         constexpr int i = decltype(i_tag)::value;
         const int row = i * RPI + rd_row;  // within the pass
         const uint4 v = *reinterpret_cast<const uint4*>(region + row * RP + rd_col);
-        *reinterpret_cast<uint4*>(out_base + (size_t)(pass * HM * 16 + row) * N * 2 + rd_col) = v;
+        // streaming store: the output is not read again by this kernel and should not push the
+        // operand slabs out of L2
+        __builtin_nontemporal_store(__builtin_bit_cast(v4i, v), reinterpret_cast<v4i*>(out_base + (size_t)(pass * HM * 16 + row) * N * 2 + rd_col));
       });
     });
     return;

@@ -74,8 +74,13 @@ __device__ __forceinline__ void mfma_acc(v4f& c, const v8i& a, const v8i& b, int
 }
 #undef KM_MFMA_ASM
 
-template <int BM, int BN, bool MX, bool SCALE_KM, int OUT>
-__global__ __launch_bounds__(256) void gemm_fp8_kernel(
+// A1: one A buffer instead of two (the A slab of step k+1 is requested at the top of step k,
+// once every wavefront holds the fragments of step k in registers, and waited for at its end).
+// Nothing stays in flight across the step boundary then, but the tile needs 3/4 of the LDS and,
+// with half the accumulators of the largest tile, two workgroups share a compute unit and fill
+// each other's waits, prologue and epilogue.
+template <int BM, int BN, bool MX, bool SCALE_KM, int OUT, bool A1>
+__global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ As, const uint8_t* __restrict__ B,
     const uint8_t* __restrict__ Bs, const float* __restrict__ sa, const float* __restrict__ sb,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N, int K) {
@@ -84,11 +89,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
   constexpr int TM = WTM / 16, TN = WTN / 16;
   constexpr int A_BYTES = BM * kStepBytes, B_BYTES = BN * kStepBytes;
   constexpr int A_LD = BM / 32, B_LD = BN / 32;  // 32 rows (4 KiB) per pass of 256 lanes
-  constexpr int kWaitAllButA = wait_vm_lgkm0(A_LD);  // all but the A_LD newest loads done
+  constexpr int kWaitAllButA = wait_vm_lgkm0(A1 ? 0 : A_LD);  // all but the A_LD newest loads done (A1: all)
   static_assert(BM % 32 == 0 && BN % 32 == 0 && TM >= 1 && TN >= 2, "tile");
   static_assert(TM * (TN - 1) >= BM / 32 + BN / 32, "every fetch pass needs its own MFMA slot");
   __shared__ __attribute__((aligned(1024))) uint8_t a_buf0[A_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t a_buf1[A_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t a_buf1[A1 ? 16 : A_BYTES];
   __shared__ __attribute__((aligned(1024))) uint8_t b_buf0[B_BYTES];
   __shared__ __attribute__((aligned(1024))) uint8_t b_buf1[B_BYTES];
 
@@ -240,7 +245,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
     constexpr int P = decltype(set_tag)::value;
     const int next = min(ks + 1, nk - 1);
     const int koff_b = __builtin_amdgcn_readfirstlane(next * kStepBytes);
-    const int koff_a = __builtin_amdgcn_readfirstlane(min(ks + 2, nk - 1) * kStepBytes);
+    const int koff_a = __builtin_amdgcn_readfirstlane(min(ks + (A1 ? 1 : 2), nk - 1) * kStepBytes);
     __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
     __syncthreads();  // every wavefront has read its A(k) fragments out of a_cur
     scale_fetch(next);
@@ -266,9 +271,10 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
           mfma_acc<0, 0>(acc[t][j], wcur, xf[j], wscale[P][t % WS], xscale[P][j % XS]);
         if constexpr (t + 1 < TN) {
           // B pass i goes after MFMA i*kBWindow/B_LD, A pass i after kBWindow + i*(kWindow-kBWindow)/A_LD
+          // (A1: everything is needed at the end of this step, so one pass per MFMA from the start)
           static_for<B_LD>([&](auto i_tag) __attribute__((always_inline)) {
             constexpr int i = decltype(i_tag)::value;
-            if constexpr (q == i * kBWindow / B_LD) {
+            if constexpr (q == (A1 ? i : i * kBWindow / B_LD)) {
               __builtin_amdgcn_sched_barrier(0);
               dma_b_pass(b_nxt, koff_b, i);
               __builtin_amdgcn_sched_barrier(0);
@@ -276,7 +282,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
           });
           static_for<A_LD>([&](auto i_tag) __attribute__((always_inline)) {
             constexpr int i = decltype(i_tag)::value;
-            if constexpr (q == kBWindow + i * (kWindow - kBWindow) / A_LD) {
+            if constexpr (q == (A1 ? B_LD + i : kBWindow + i * (kWindow - kBWindow) / A_LD)) {
               __builtin_amdgcn_sched_barrier(0);
               dma_a_pass(a_cur, koff_a, i);
               __builtin_amdgcn_sched_barrier(0);
@@ -304,7 +310,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
   dma_a(a_buf0, 0);
   dma_b(b_buf0, 0);
   scale_fetch(0);
-  dma_a(a_buf1, min(1, nk - 1));
+  if constexpr (!A1) dma_a(a_buf1, min(1, nk - 1));
   __builtin_amdgcn_s_waitcnt(kWaitVm0);
   __syncthreads();
   scale_commit(set0_t{}, 0xFFFFFFFFu);
@@ -315,8 +321,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
   // two steps per trip, one per buffer parity; an odd step count is padded with a zero-scaled step
   const int nsteps = (nk + 1) & ~1;
   for (int ks = 0; ks < nsteps; ks += 2) {
-    step(a_buf0, a_buf1, b_buf0, b_buf1, ks, set0_t{});
-    step(a_buf1, a_buf0, b_buf1, b_buf0, ks + 1, set1_t{});
+    step(a_buf0, A1 ? a_buf0 : a_buf1, b_buf0, b_buf1, ks, set0_t{});
+    step(A1 ? a_buf0 : a_buf1, a_buf0, b_buf1, b_buf0, ks + 1, set1_t{});
   }
   __builtin_amdgcn_s_waitcnt(kWaitVm0);  // the last (clamped) A prefetch must land before LDS is reused
 
@@ -329,7 +335,12 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(
   // epilogue: bias (and the per-tensor scales) on the fp32 accumulator, one rounding
   float post = 1.0f;
   if constexpr (!MX) post = sa[0] * sb[0];
-  store_tile<BM, BN, OUT, !MX>(acc, post, nullptr, bias, C, M, N, m0, n0, a_buf0, a_buf1, b_buf0, b_buf1);
+  if constexpr (A1) {
+    static_assert(B_BYTES / 2 >= (BM < BN ? BM : BN) * 128, "epilogue staging in the halves of the B buffers");
+    store_tile<BM, BN, OUT, !MX>(acc, post, nullptr, bias, C, M, N, m0, n0, b_buf0, b_buf0 + B_BYTES / 2, b_buf1, b_buf1 + B_BYTES / 2);
+  } else {
+    store_tile<BM, BN, OUT, !MX>(acc, post, nullptr, bias, C, M, N, m0, n0, a_buf0, a_buf1, b_buf0, b_buf1);
+  }
 }
 
 struct GemmConfig {
@@ -346,12 +357,12 @@ static const GemmConfig kGemmConfigs[] = {
 };
 constexpr int kNumGemmConfigs = sizeof(kGemmConfigs) / sizeof(kGemmConfigs[0]);
 
-template <int BM, int BN, bool MX, bool SCALE_KM, int OUT>
+template <int BM, int BN, bool MX, bool SCALE_KM, int OUT, bool A1 = false>
 static int launch_gemm(const void* a, const void* as, const void* b, const void* bs, const float* sa,
                        const float* sb, const void* bias, void* c, int M, int N, int K,
                        hipStream_t st) {
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  hipLaunchKernelGGL((gemm_fp8_kernel<BM, BN, MX, SCALE_KM, OUT>), dim3(tiles), dim3(256), 0, st,
+  hipLaunchKernelGGL((gemm_fp8_kernel<BM, BN, MX, SCALE_KM, OUT, A1>), dim3(tiles), dim3(256), 0, st,
                      (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b, (const uint8_t*)bs, sa, sb,
                      (const uint16_t*)bias, (uint16_t*)c, M, N, K);
   return km_check_launch("km_gemm");
@@ -363,7 +374,7 @@ static int dispatch_config(int config, const void* a, const void* as, const void
                            int K, hipStream_t st) {
   switch (config) {
     case 0: return launch_gemm<256, 256, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
-    case 1: return launch_gemm<128, 256, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
+    case 1: return launch_gemm<128, 256, MX, SCALE_KM, OUT, true>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
     case 2: return launch_gemm<256, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
     case 3: return launch_gemm<128, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
     case 4: return launch_gemm<64, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
@@ -405,7 +416,7 @@ int gemm_num_configs() { return kNumGemmConfigs; }
 int gemm_config_desc(int config, char* buf, int len) {
   if (config < 0 || config >= kNumGemmConfigs) return km_fail(KM_ERR_ARG, "config out of range");
   const GemmConfig& c = kGemmConfigs[config];
-  snprintf(buf, len, "bm=%d,bn=%d,bk=128,waves=4", c.bm, c.bn);
+  snprintf(buf, len, "bm=%d,bn=%d,bk=128,waves=4,wg_per_cu=%d", c.bm, c.bn, config == 1 || config >= 3 ? 2 : 1);
   return KM_OK;
 }
 

@@ -79,8 +79,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   const int r16 = lane & 15, g = lane >> 4;
   const int nk = (KC + kWoStepElems - 1) / kWoStepElems;
 
-  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(A) + (size_t)m0 * KC, 0, (int)min((int64_t)(M - m0) * KC * 2, (int64_t)0x7FFFFFFF), 0x00020000);
+  const v4i a_rsrc = raw_rsrc(A + (size_t)m0 * KC, (uint32_t)min((int64_t)(M - m0) * KC * 2, (int64_t)0x7FFFFFFF));
   const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint8_t*>(Q) + (size_t)n0 * KC, 0, (int)min((int64_t)(NO - n0) * KC, (int64_t)0x7FFFFFFF), 0x00020000);
   // staging map of a pass: 8 lanes per row; 16 lanes cover rows r and r+8 (one LDS line)
@@ -106,7 +105,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   auto dma_a_pass = [&](uint8_t* buf, int ks, int i) __attribute__((always_inline)) {
     const int col = ks * kWoStepElems + a_chunk * 8;
     const int voff = col < KC ? ((srow + i * 32) * KC + col) * 2 : kOob;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(buf + i * 4096 + wave * 1024), 16, voff, 0, 0, 0);
+    hidden_dma_b128(a_rsrc, lds_offset(buf) + i * 4096 + wave * 1024, voff, 0);  // waited for at the end of the step
   };
   auto q_load_pass = [&](int ks, int i) __attribute__((always_inline)) {
     const int col = ks * kWoStepElems + q_chunk * 8;
