@@ -74,6 +74,65 @@ __device__ __forceinline__ uint2 encode8(const float (&f)[8], float inv) {
   return make_uint2(lo, hi);
 }
 
+// ---- hardware e4m3 conversion ----------------------------------------------------------------
+// V_CVT_SCALEF32_PK_FP8_{BF16,F16,F32} divide by the power of two in the exponent field of the
+// scale operand, round once to nearest even and, with MODE.FP16_OVFL set, saturate at +-448: the
+// reference's clamp((x * 2^-e)).to(e4m3) in one instruction per two elements, checked against
+// the software encoder on every 16-bit input pattern and every scale byte a block can get.
+// The one difference is NaN, which the instruction turns into 0xFF whatever the sign;
+// nan_fix() restores 0x7F | sign.
+typedef short v2s __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef unsigned short v2us __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void saturating_conversions() {
+  asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 1");  // FP16_OVFL, per wavefront
+}
+// 16-bit absolute-value bits above which a pattern is a NaN
+template <int DT>
+constexpr uint32_t inf16() { return DT == KM_BF16 ? 0x7F80u : 0x7C00u; }
+// fp32 bits of a non-negative 16-bit pattern (monotonic, NaN patterns stay above infinity)
+template <int DT>
+__device__ __forceinline__ uint32_t widen_bits(uint32_t h) {
+  if constexpr (DT == KM_BF16) return h << 16;
+  else return f32_bits(__half2float(__ushort_as_half((unsigned short)h)));
+}
+// four codes from two dwords of packed 16-bit values (a.lo, a.hi, b.lo, b.hi)
+template <int DT>
+__device__ __forceinline__ uint32_t cvt4(uint32_t a, uint32_t b, float scale) {
+  v2s r = {0, 0};
+  if constexpr (DT == KM_BF16) {
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(r, __builtin_bit_cast(v2bf, a), scale, false);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(r, __builtin_bit_cast(v2bf, b), scale, true);
+  } else {
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, __builtin_bit_cast(v2h, a), scale, false);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, __builtin_bit_cast(v2h, b), scale, true);
+  }
+  return __builtin_bit_cast(uint32_t, r);
+}
+// four codes from four fp32 values
+__device__ __forceinline__ uint32_t cvt4_f32(float a, float b, float c, float d, float scale) {
+  v2s r = {0, 0};
+  r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(r, a, b, scale, false);
+  r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(r, c, d, scale, true);
+  return __builtin_bit_cast(uint32_t, r);
+}
+// codes of the two 16-bit values in `h` (bytes `shift`, `shift`+8 of `codes`): NaN -> 0x7F | sign
+template <int DT>
+__device__ __forceinline__ uint32_t nan_fix(uint32_t codes, uint32_t h, int shift) {
+  if ((h & 0x7FFFu) > inf16<DT>()) codes = (codes & ~(0xFFu << shift)) | ((0x7Fu | ((h >> 8) & 0x80u)) << shift);
+  if (((h >> 16) & 0x7FFFu) > inf16<DT>()) codes = (codes & ~(0xFF00u << shift)) | ((0x7Fu | ((h >> 24) & 0x80u)) << (shift + 8));
+  return codes;
+}
+// largest 16-bit absolute-value pattern of the eight values of one 128-bit load
+__device__ __forceinline__ uint32_t amax16x8(const uint4& raw) {
+  const v2us a = __builtin_bit_cast(v2us, raw.x & 0x7FFF7FFFu), b = __builtin_bit_cast(v2us, raw.y & 0x7FFF7FFFu);
+  const v2us c = __builtin_bit_cast(v2us, raw.z & 0x7FFF7FFFu), d = __builtin_bit_cast(v2us, raw.w & 0x7FFF7FFFu);
+  const v2us m = __builtin_elementwise_max(__builtin_elementwise_max(a, b), __builtin_elementwise_max(c, d));
+  return m.x > m.y ? m.x : m.y;
+}
+
 // ---- rows: lane = 8 consecutive elements, quad = one block of 32 --------------------------
 // Group g (8 elements) of row g / groups_per_row; outputs are flat because q and the
 // scales are contiguous row-major. UNROLL independent 128-bit loads are in flight per lane.
@@ -96,6 +155,7 @@ template <int DT, bool PACK4>
 __global__ __launch_bounds__(kRowsThreads) void quant_mx_rows(
     const uint16_t* __restrict__ x, int64_t ld, uint32_t groups_per_row, uint64_t ngroups, uint32_t rows,
     uint8_t* __restrict__ q, uint8_t* __restrict__ scales, uint8_t* __restrict__ scales_km) {
+  saturating_conversions();
   const uint64_t base = (uint64_t)blockIdx.x * (kRowsThreads * kRowsUnroll) + threadIdx.x;
   const bool dense = ld == (int64_t)groups_per_row * 8;
   uint4 raw[kRowsUnroll];
@@ -117,10 +177,14 @@ __global__ __launch_bounds__(kRowsThreads) void quant_mx_rows(
 #pragma unroll
   for (int u = 0; u < kRowsUnroll; ++u) {
     const uint64_t g = base + (uint64_t)u * kRowsThreads;
-    float f[8];
-    widen8<DT>(raw[u], f);
-    const uint32_t biased = mx_biased_exponent(quad_max(amax_bits8(f)));
-    const uint2 codes = encode8(f, mx_inverse_scale(biased));
+    const uint32_t m16 = amax16x8(raw[u]);
+    const uint32_t biased = mx_biased_exponent(quad_max(widen_bits<DT>(m16)));
+    const float sc = bits_f32(biased << 23);  // 2^(biased - 127) as the conversion's scale operand
+    uint2 codes = make_uint2(cvt4<DT>(raw[u].x, raw[u].y, sc), cvt4<DT>(raw[u].z, raw[u].w, sc));
+    if (m16 > inf16<DT>()) {  // a NaN among these eight (rare)
+      codes.x = nan_fix<DT>(nan_fix<DT>(codes.x, raw[u].x, 0), raw[u].y, 16);
+      codes.y = nan_fix<DT>(nan_fix<DT>(codes.y, raw[u].z, 0), raw[u].w, 16);
+    }
     if constexpr (PACK4) {
       const uint32_t four = gather4_stride4(biased);
       if (g < ngroups) {
@@ -161,6 +225,7 @@ __global__ __launch_bounds__(kColsThreads) void quant_mx_cols(
   const int64_t r0 = (int64_t)blockIdx.y * kColsTR;
   const int64_t c0 = (int64_t)blockIdx.x * kColsTC;
   const int tid = threadIdx.x;
+  saturating_conversions();
   // stage: 8 lanes cover one 128-byte row segment
   {
     const int cg = tid & 7;   // 8-element group within the row segment
@@ -191,27 +256,26 @@ __global__ __launch_bounds__(kColsThreads) void quant_mx_cols(
   uint32_t w[32];
 #pragma unroll
   for (int i = 0; i < 32; ++i) w[i] = col[i * kColsPitch];
-  uint32_t m0 = 0, m1 = 0;
-  float f0[32], f1[32];
+  // the two columns of the pair: low and high halves of the 32 dwords
+  uint32_t mm = 0;
 #pragma unroll
   for (int i = 0; i < 32; ++i) {
-    f0[i] = widen<DT>(w[i] & 0xFFFFu);
-    f1[i] = widen<DT>(w[i] >> 16);
-    const uint32_t a0 = f32_bits(f0[i]) & kAbsMask, a1 = f32_bits(f1[i]) & kAbsMask;
-    m0 = a0 > m0 ? a0 : m0;
-    m1 = a1 > m1 ? a1 : m1;
+    const v2us a = __builtin_bit_cast(v2us, w[i] & 0x7FFF7FFFu), m = __builtin_bit_cast(v2us, mm);
+    mm = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, m));
   }
-  const uint32_t b0 = mx_biased_exponent(m0), b1 = mx_biased_exponent(m1);
-  const float i0 = mx_inverse_scale(b0), i1 = mx_inverse_scale(b1);
+  const uint32_t m0 = mm & 0xFFFFu, m1 = mm >> 16;
+  const uint32_t b0 = mx_biased_exponent(widen_bits<DT>(m0)), b1 = mx_biased_exponent(widen_bits<DT>(m1));
+  const float s0 = bits_f32(b0 << 23), s1 = bits_f32(b1 << 23);
   uint32_t o0[8], o1[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    o0[j] = o1[j] = 0;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      o0[j] |= e4m3_encode(f0[4 * j + t] * i0) << (8 * t);
-      o1[j] |= e4m3_encode(f1[4 * j + t] * i1) << (8 * t);
-    }
+    // rows 4j .. 4j+3 of each column: regroup the halves so that a conversion sees one column
+    const uint32_t lo01 = __builtin_amdgcn_perm(w[4 * j + 1], w[4 * j], 0x05040100u), hi01 = __builtin_amdgcn_perm(w[4 * j + 1], w[4 * j], 0x07060302u);
+    const uint32_t lo23 = __builtin_amdgcn_perm(w[4 * j + 3], w[4 * j + 2], 0x05040100u), hi23 = __builtin_amdgcn_perm(w[4 * j + 3], w[4 * j + 2], 0x07060302u);
+    o0[j] = cvt4<DT>(lo01, lo23, s0);
+    o1[j] = cvt4<DT>(hi01, hi23, s1);
+    if (m0 > inf16<DT>()) o0[j] = nan_fix<DT>(nan_fix<DT>(o0[j], lo01, 0), lo23, 16);
+    if (m1 > inf16<DT>()) o1[j] = nan_fix<DT>(nan_fix<DT>(o1[j], hi01, 0), hi23, 16);
   }
   uint4* d0 = reinterpret_cast<uint4*>(q_t + c * rows + rb);
   d0[0] = make_uint4(o0[0], o0[1], o0[2], o0[3]);
