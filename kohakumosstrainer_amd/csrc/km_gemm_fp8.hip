@@ -229,8 +229,9 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
     return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
   // One K step with parity P: A(k) is already in registers, B(k) is in b_cur. Fetches B(k+1)
-  // into b_nxt and A(k+2) into a_cur (its A(k) was consumed during the step before; the
-  // barrier at the top makes sure by every wavefront), multiplies, waits for B(k+1) only,
+  // into b_nxt (free since the barrier in the last group of the step before) and A(k+2) into
+  // a_cur (its A(k) was consumed during the step before; a barrier just ahead of the first A
+  // pass makes sure by every wavefront), multiplies, waits for B(k+1) only,
   // and reads the first fragments of step k+1 (A(k+1) from a_nxt was issued a step earlier)
   // during the last MFMA group; each fragment register is reloaded one MFMA after the last
   // MFMA that read it. The scales of step k+1 are committed to set P^1.
@@ -246,8 +247,6 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
     const int next = min(ks + 1, nk - 1);
     const int koff_b = __builtin_amdgcn_readfirstlane(next * kStepBytes);
     const int koff_a = __builtin_amdgcn_readfirstlane(min(ks + (A1 ? 1 : 2), nk - 1) * kStepBytes);
-    __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
-    __syncthreads();  // every wavefront has read its A(k) fragments out of a_cur
     scale_fetch(next);
     __builtin_amdgcn_sched_barrier(0);
     static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
@@ -284,6 +283,13 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
             constexpr int i = decltype(i_tag)::value;
             if constexpr (q == (A1 ? B_LD + i : kBWindow + i * (kWindow - kBWindow) / A_LD)) {
               __builtin_amdgcn_sched_barrier(0);
+              if constexpr (i == 0) {
+                // a_cur still holds A(k): its fragments were read at the end of the step before.
+                // Waiting for them here, not at the top of the step, costs nothing: they arrived
+                // long ago, and every wavefront must have them before the slab is overwritten.
+                __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+                __syncthreads();
+              }
               dma_a_pass(a_cur, koff_a, i);
               __builtin_amdgcn_sched_barrier(0);
             }
@@ -324,7 +330,7 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
     step(a_buf0, A1 ? a_buf0 : a_buf1, b_buf0, b_buf1, ks, set0_t{});
     step(A1 ? a_buf0 : a_buf1, a_buf0, b_buf1, b_buf0, ks + 1, set1_t{});
   }
-  __builtin_amdgcn_s_waitcnt(kWaitVm0);  // the last (clamped) A prefetch must land before LDS is reused
+  __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));  // the last (clamped) prefetches and fragment reads must be done before LDS is reused
 
   // the MFMAs above are opaque to the compiler's hazard handling: give the last ones time to
   // retire before the accumulators are read
