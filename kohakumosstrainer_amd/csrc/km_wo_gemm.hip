@@ -42,18 +42,51 @@ __device__ __forceinline__ void mfma16(v4f& c, const v4i& a, const v4i& b) {
 
 // 8 codes (two dwords) -> 8 values of the activation type (four dwords); `s` scales them in
 // fp32 before the single rounding (dgrad), or is 1 (forward: the conversion is exact)
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+
+// four e4m3 codes of one dword -> four fp32 (V_CVT_PK_F32_FP8, two codes per instruction)
+__device__ __forceinline__ void e4m3x4_to_f32(uint32_t w, float (&f)[4]) {
+  const v2f lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+  f[0] = lo.x; f[1] = lo.y; f[2] = hi.x; f[3] = hi.y;
+}
+// four e4m3 codes -> two dwords of the activation type: every e4m3 value is exact in bf16 and
+// f16, so the scaled conversion with scale 1 is the whole job (two codes per instruction)
+template <int DT>
+__device__ __forceinline__ uint2 e4m3x4_to_16(uint32_t w) {
+  if constexpr (DT == KM_BF16)
+    return make_uint2(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false)),
+                      __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true)));
+  else
+    return make_uint2(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false)),
+                      __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true)));
+}
+
 template <int DT, int QF, bool SCALE>
 __device__ __forceinline__ uint4 widen_codes(uint2 raw, const float (&s)[8]) {
-  float f[8];
-  const uint32_t w[2] = {raw.x, raw.y};
+  if constexpr (QF == KM_Q_E4M3 && !SCALE) {
+    const uint2 lo = e4m3x4_to_16<DT>(raw.x), hi = e4m3x4_to_16<DT>(raw.y);
+    return make_uint4(lo.x, lo.y, hi.x, hi.y);
+  } else {
+    float f[8];
+    if constexpr (QF == KM_Q_E4M3) {
+      float a[4], b[4];
+      e4m3x4_to_f32(raw.x, a);
+      e4m3x4_to_f32(raw.y, b);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const uint32_t byte = (w[i >> 2] >> (8 * (i & 3))) & 0xFFu;
-    if constexpr (QF == KM_Q_INT8) f[i] = (float)(int)(int8_t)byte;
-    else f[i] = e4m3_decode(byte);
-    if constexpr (SCALE) f[i] *= s[i];
+      for (int i = 0; i < 4; ++i) { f[i] = a[i]; f[4 + i] = b[i]; }
+    } else {
+      const uint32_t w[2] = {raw.x, raw.y};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] = (float)(int)(int8_t)((w[i >> 2] >> (8 * (i & 3))) & 0xFFu);
+    }
+    if constexpr (SCALE) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] *= s[i];
+    }
+    return make_uint4(pack2<DT>(f[0], f[1]), pack2<DT>(f[2], f[3]), pack2<DT>(f[4], f[5]), pack2<DT>(f[6], f[7]));
   }
-  return make_uint4(pack2<DT>(f[0], f[1]), pack2<DT>(f[2], f[3]), pack2<DT>(f[4], f[5]), pack2<DT>(f[6], f[7]));
 }
 
 template <int BM, int BN, int DT, int QF, bool DGRAD>

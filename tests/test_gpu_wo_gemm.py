@@ -124,3 +124,20 @@ def test_argument_errors():
     with pytest.raises(native.KernelError):
         native.wo_gemm_fwd(x, q, s, None, 99)
     assert native.wo_gemm_fwd(x[:0], q, s, None).shape == (0, 16)
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+def test_every_e4m3_code_widens_exactly(dtype):
+    """Identity activations read the widened weight back: forward must return every finite
+    e4m3 code's exact value (all are representable in bf16 and f16), dgrad the once-rounded
+    scaled value. (The two NaN codes are left out: a NaN weight poisons every sum it is in.)"""
+    codes = torch.arange(256, dtype=torch.uint8)
+    codes[0x7F] = 0
+    codes[0xFF] = 0x80
+    q = torch.cat([codes.repeat(2, 1), codes.flip(0).repeat(2, 1)], 0).contiguous().view(torch.float8_e4m3fn)  # [N=4, K=256]
+    scale = torch.tensor([1.0, 0.37, 3.0, 1e-3])
+    eye = torch.eye(256, dtype=dtype)
+    y = native.wo_gemm_fwd(eye.cuda(), q.cuda(), torch.ones(4).cuda(), None, 0).cpu()  # [256, 4] = W^T
+    assert torch.equal(y.float(), q.float().t())
+    dx = native.wo_gemm_dgrad(torch.eye(4, dtype=dtype).cuda(), q.cuda(), scale.cuda(), 0).cpu()  # [4, 256] = round(W * s)
+    assert torch.equal(dx, (q.float() * scale[:, None]).to(dtype))
