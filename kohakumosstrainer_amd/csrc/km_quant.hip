@@ -211,9 +211,9 @@ __global__ __launch_bounds__(kRowsThreads) void quant_mx_rows(
 // TR x TC tile in LDS with 128-bit row loads, then each lane owns two adjacent columns of one
 // 32-row block: it reads 32 dwords down the tile, reduces in registers and writes two
 // 32-byte runs of q_t.
-constexpr int kColsThreads = 256;
+constexpr int kColsThreads = 512;
 constexpr int kColsTR = 256;  // rows of x per tile (8 blocks)
-constexpr int kColsTC = 64;   // columns of x per tile
+constexpr int kColsTC = 128;  // columns of x per tile: 256-byte row segments
 constexpr int kColsPitch = kColsTC / 2 + 4;  // dwords per staged row (16-byte aligned rows)
 constexpr int kColsSkew = 8;  // extra dwords after each 32 rows: spreads the 8 blocks over banks
 
@@ -226,10 +226,12 @@ __global__ __launch_bounds__(kColsThreads) void quant_mx_cols(
   const int64_t c0 = (int64_t)blockIdx.x * kColsTC;
   const int tid = threadIdx.x;
   saturating_conversions();
-  // stage: 8 lanes cover one 128-byte row segment
+  // stage: 16 lanes cover one 256-byte row segment
   {
-    const int cg = tid & 7;   // 8-element group within the row segment
-    const int rr = tid >> 3;  // 0..31
+    constexpr int kLanesPerRow = kColsTC / 8;
+    static_assert(kColsThreads / kLanesPerRow == 32, "a staging pass covers 32 rows");
+    const int cg = tid % kLanesPerRow;  // 8-element group within the row segment
+    const int rr = tid / kLanesPerRow;  // 0..31
     uint4 raw[kColsTR / 32];
 #pragma unroll
     for (int i = 0; i < kColsTR / 32; ++i) {
@@ -248,7 +250,7 @@ __global__ __launch_bounds__(kColsThreads) void quant_mx_cols(
   // lane -> (block of 32 rows, column pair); blocks vary fastest so a wave writes runs of
   // consecutive bytes of q_t rows
   const int blk = tid & 7;
-  const int pair = tid >> 3;  // 0..31
+  const int pair = tid >> 3;  // 0 .. kColsTC / 2 - 1
   const int64_t rb = r0 + blk * 32;
   const int64_t c = c0 + pair * 2;
   if (rb >= rows || c >= cols) return;
