@@ -80,7 +80,7 @@ def cpu_baseline(x, wq, ws, bias):
 
 
 def other_configs(dev, reps):
-    """Device time of the other kernels of the path at their BASELINE shapes (event-timed,
+    """Device time of the other kernels of the path at their benchmark shapes (event-timed,
     back to back): weight-only int8 / e4m3 GEMMs and the frozen-base MXFP8 forward + input
     gradient of the adapter-training shape."""
     from kohakumosstrainer_amd import native
@@ -228,7 +228,7 @@ def main():
         "dtype": "fp8_e4m3 (E8M0 block scales), fp32 accumulate, bf16 out",
         "data": "synthetic",
         "config": {
-            "workload": f"MXFP8 fused-QKV linear forward M={M} K={K} N={N}: per-call activation quantizer + block-scaled GEMM + bias, bf16 out (BASELINE configs[3]); quantizer alone on bf16 [{M},{K}] row- and column-wise (configs[2])",
+            "workload": f"MXFP8 fused-QKV linear forward M={M} K={K} N={N}: per-call activation quantizer + block-scaled GEMM + bias, bf16 out (benchmark configs[3]); quantizer alone on bf16 [{M},{K}] row- and column-wise (configs[2])",
             "gemm_tile_config": config,
             "gemm_tile_configs_ms": tried,
         },
