@@ -16,7 +16,8 @@ How each function is pinned (independently of its own formula):
   formats.mx_biased_exponent   definition "smallest e >= -127 with 2^e*448 >= amax"
                                by a loop in exact arithmetic; the reference tests'
                                known answers (amax 1.75 -> 119, 1.75(1+2^-7) -> 120,
-                               all-zero block -> 19, 448*2^-130 -> 0)
+                               all-zero block -> 19, and so 448*2^-130: the 1e-30 amax
+                               floor makes byte 0 unreachable)
   formats.fp32_scale           correctly rounded fp32 division via numpy float32
   formats.quantize / dequantize  block-by-block application of the two above; q*scale
                                per element in fp64
