@@ -63,6 +63,14 @@ int km_scales_pack(const void *scales, int64_t rows, int64_t cols, void *out, vo
 int km_quant_tensor(const void *x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,
                     int dtype, void *q, float *scale_out, uint32_t *amax_workspace, void *stream);
 
+/* Per-row e4m3 quantizer: scale_out[r] = max(amax of row r, 1e-12) / 448 (IEEE division),
+ * q[r, :] = e4m3(clamp(x[r, :] / scale_out[r])) (IEEE division, clamp to +-448, one rounding).
+ * Any strides and cols; unit-stride rows with cols % 8 == 0 take the vectorized kernel.
+ * Replaces fp8.formats.quantize(x, "row") (src/kohakumoss_kernels/fp8/formats.py:80-82) and
+ * Triton quantize_rows (backends/triton/fp8/quantize.py:64-84,151-158). */
+int km_quant_rows(const void *x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,
+                  int dtype, void *q, float *scale_out, void *stream);
+
 /* C[M,N] = (A .* 2^(a_scale-127)) (B .* 2^(b_scale-127))^T + bias, A [M,K] and B [N,K] e4m3fn
  * row-major (K contiguous), scales E8M0 bytes, both in the layout scale_layout names
  * (KM_SCALES_ROWMAJOR: [M,K/32] / [N,K/32]; KM_SCALES_PACKED: see km_scales_pack), fp32 accumulation
@@ -80,6 +88,14 @@ int km_gemm_mx(const void *a, const void *a_scale, const void *b, const void *b_
 int km_gemm_fp8_tensor(const void *a, const float *sa, const void *b, const float *sb,
                        const void *bias, void *c, int64_t M, int64_t N, int64_t K, int out_dtype,
                        int config, void *stream);
+
+/* Per-row fp8 GEMM: C[m,n] = (A B^T)[m,n] * (sa[m] * sb[n]) + bias[n], sa [M] and sb [N] device
+ * fp32 vectors (sb 16-byte aligned). Replaces Triton scaled_mm for the row recipe
+ * (backends/triton/fp8/gemm.py:66-105,187-202) and torch._scaled_mm with row-wise scales
+ * (backends/triton/fp8/linear.py:130-136). K % 128 == 0. */
+int km_gemm_fp8_rows(const void *a, const float *sa, const void *b, const float *sb,
+                     const void *bias, void *c, int64_t M, int64_t N, int64_t K, int out_dtype,
+                     int config, void *stream);
 
 /* Weight-only forward: y[M,N] = (x[M,K] @ q[N,K]^T) * scale[N] + bias[N]; q int8 or e4m3fn
  * widened exactly to the activation dtype in registers, fp32 accumulation, scale and bias on

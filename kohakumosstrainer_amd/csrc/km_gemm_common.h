@@ -118,12 +118,12 @@ __device__ __forceinline__ uint32_t hidden_load_b32(const v4i& rsrc, int voffset
 
 // Epilogue of a 2 x 2 wavefront grid over a BM x BN tile of 16x16 MFMA tiles whose rows are
 // output columns: lane (r16 = lane%16, g = lane/16) of tile (t, j) holds
-// C[m0+wm+j*16+r16][n0+wn+t*16+4g .. +3]. Computes acc * post * col_scale[n] + bias[n] in fp32,
-// rounds once to the 16-bit output type. `bufs` are four LDS buffers of at least
+// C[m0+wm+j*16+r16][n0+wn+t*16+4g .. +3]. Computes acc * post * row_scale[m] * col_scale[n] +
+// bias[n] in fp32 (either scale vector may be null), rounds once to the 16-bit output type. `bufs` are four LDS buffers of at least
 // `buf_bytes` each, free for staging (one per wavefront).
 template <int BM, int BN, int OUT, bool SCALED>
-__device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float post, const float* __restrict__ col_scale,
-                                           const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N,
+__device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float post, const float* __restrict__ row_scale,
+                                           const float* __restrict__ col_scale, const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N,
                                            int m0, int n0, uint8_t* buf0, uint8_t* buf1, uint8_t* buf2, uint8_t* buf3) {
   constexpr int WTM = BM / 2, WTN = BN / 2, TM = WTM / 16, TN = WTN / 16;
   const int lane = threadIdx.x & 63;
@@ -131,8 +131,8 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
   const int wm = (wave >> 1) * WTM, wn = (wave & 1) * WTN;
   const int r16 = lane & 15, g = lane >> 4;
   const bool has_bias = bias != nullptr;
-  auto value = [&](float a, float cs, float b) __attribute__((always_inline)) {
-    if constexpr (SCALED) return a * (post * cs) + b;
+  auto value = [&](float a, float rs, float cs, float b) __attribute__((always_inline)) {
+    if constexpr (SCALED) return a * (rs * cs) + b;
     else return a + b;
   };
   if (m0 + BM <= M && n0 + BN <= N && (N & 7) == 0) {
@@ -166,6 +166,9 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
         bv[t][2] = unpack1<OUT>(braw.y & 0xFFFFu); bv[t][3] = unpack1<OUT>(braw.y >> 16);
       }
     });
+    float rs[TM];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) rs[j] = row_scale != nullptr ? post * row_scale[m0 + wm + j * 16 + r16] : post;
     uint8_t* out_base = reinterpret_cast<uint8_t*>(C) + ((size_t)(m0 + wm) * N + n0 + wn) * 2;
     const int rd_row = lane / LPR, rd_col = (lane % LPR) * 16;
     static_for<TM / HM>([&](auto p_tag) __attribute__((always_inline)) {
@@ -177,7 +180,7 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
           constexpr int t = decltype(t_tag)::value;
           float o[4];
 #pragma unroll
-          for (int v = 0; v < 4; ++v) o[v] = value(acc[t][j][v], cs[t][v], bv[t][v]);
+          for (int v = 0; v < 4; ++v) o[v] = value(acc[t][j][v], rs[j], cs[t][v], bv[t][v]);
           *reinterpret_cast<uint2*>(region + (jj * 16 + r16) * RP + (t * 16 + 4 * g) * 2) =
               make_uint2(pack2<OUT>(o[0], o[1]), pack2<OUT>(o[2], o[3]));
         });
@@ -208,9 +211,10 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
     for (int j = 0; j < TM; ++j) {
       const int m = m0 + wm + j * 16 + r16;
       if (m >= M || n >= N) continue;
+      const float rs = row_scale != nullptr ? post * row_scale[m] : post;
       float o[4];
 #pragma unroll
-      for (int v = 0; v < 4; ++v) o[v] = value(acc[t][j][v], cs[v], bv[v]);
+      for (int v = 0; v < 4; ++v) o[v] = value(acc[t][j][v], rs, cs[v], bv[v]);
       uint16_t* dst = C + (size_t)m * N + n;
       if (vec_ok && n + 3 < N) {
         *reinterpret_cast<uint2*>(dst) = make_uint2(pack2<OUT>(o[0], o[1]), pack2<OUT>(o[2], o[3]));

@@ -83,7 +83,7 @@ template <int BM, int BN, bool MX, bool SCALE_KM, int OUT, bool A1>
 __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ As, const uint8_t* __restrict__ B,
     const uint8_t* __restrict__ Bs, const float* __restrict__ sa, const float* __restrict__ sb,
-    const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N, int K) {
+    const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N, int K, int scale_vectors) {
   constexpr int NT = 256;
   constexpr int WTM = BM / 2, WTN = BN / 2;
   constexpr int TM = WTM / 16, TN = WTN / 16;
@@ -340,12 +340,20 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
 
   // epilogue: bias (and the per-tensor scales) on the fp32 accumulator, one rounding
   float post = 1.0f;
-  if constexpr (!MX) post = sa[0] * sb[0];
+  const float *row_scale = nullptr, *col_scale = nullptr;
+  if constexpr (!MX) {
+    if (scale_vectors) {
+      row_scale = sa;
+      col_scale = sb;
+    } else {
+      post = sa[0] * sb[0];
+    }
+  }
   if constexpr (A1) {
     static_assert(B_BYTES / 2 >= (BM < BN ? BM : BN) * 128, "epilogue staging in the halves of the B buffers");
-    store_tile<BM, BN, OUT, !MX>(acc, post, nullptr, bias, C, M, N, m0, n0, b_buf0, b_buf0 + B_BYTES / 2, b_buf1, b_buf1 + B_BYTES / 2);
+    store_tile<BM, BN, OUT, !MX>(acc, post, row_scale, col_scale, bias, C, M, N, m0, n0, b_buf0, b_buf0 + B_BYTES / 2, b_buf1, b_buf1 + B_BYTES / 2);
   } else {
-    store_tile<BM, BN, OUT, !MX>(acc, post, nullptr, bias, C, M, N, m0, n0, a_buf0, a_buf1, b_buf0, b_buf1);
+    store_tile<BM, BN, OUT, !MX>(acc, post, row_scale, col_scale, bias, C, M, N, m0, n0, a_buf0, a_buf1, b_buf0, b_buf1);
   }
 }
 
@@ -365,25 +373,25 @@ constexpr int kNumGemmConfigs = sizeof(kGemmConfigs) / sizeof(kGemmConfigs[0]);
 
 template <int BM, int BN, bool MX, bool SCALE_KM, int OUT, bool A1 = false>
 static int launch_gemm(const void* a, const void* as, const void* b, const void* bs, const float* sa,
-                       const float* sb, const void* bias, void* c, int M, int N, int K,
+                       const float* sb, const void* bias, void* c, int M, int N, int K, int scale_vectors,
                        hipStream_t st) {
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   hipLaunchKernelGGL((gemm_fp8_kernel<BM, BN, MX, SCALE_KM, OUT, A1>), dim3(tiles), dim3(256), 0, st,
                      (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b, (const uint8_t*)bs, sa, sb,
-                     (const uint16_t*)bias, (uint16_t*)c, M, N, K);
+                     (const uint16_t*)bias, (uint16_t*)c, M, N, K, scale_vectors);
   return km_check_launch("km_gemm");
 }
 
 template <bool MX, bool SCALE_KM, int OUT>
 static int dispatch_config(int config, const void* a, const void* as, const void* b, const void* bs,
                            const float* sa, const float* sb, const void* bias, void* c, int M, int N,
-                           int K, hipStream_t st) {
+                           int K, int scale_vectors, hipStream_t st) {
   switch (config) {
-    case 0: return launch_gemm<256, 256, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
-    case 1: return launch_gemm<128, 256, MX, SCALE_KM, OUT, true>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
-    case 2: return launch_gemm<256, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
-    case 3: return launch_gemm<128, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
-    case 4: return launch_gemm<64, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, st);
+    case 0: return launch_gemm<256, 256, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
+    case 1: return launch_gemm<128, 256, MX, SCALE_KM, OUT, true>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
+    case 2: return launch_gemm<256, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
+    case 3: return launch_gemm<128, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
+    case 4: return launch_gemm<64, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
   }
   return km_fail(KM_ERR_ARG, "km_gemm: unknown config");
 }
@@ -444,11 +452,11 @@ extern "C" int km_gemm_mx(const void* a, const void* a_scale, const void* b, con
   hipStream_t st = (hipStream_t)stream;
   const bool km = scale_layout == KM_SCALES_PACKED;
   if (out_dtype == KM_BF16) {
-    if (km) return dispatch_config<true, true, KM_BF16>(config, a, a_scale, b, b_scale, nullptr, nullptr, bias, c, (int)M, (int)N, (int)K, st);
-    return dispatch_config<true, false, KM_BF16>(config, a, a_scale, b, b_scale, nullptr, nullptr, bias, c, (int)M, (int)N, (int)K, st);
+    if (km) return dispatch_config<true, true, KM_BF16>(config, a, a_scale, b, b_scale, nullptr, nullptr, bias, c, (int)M, (int)N, (int)K, 0, st);
+    return dispatch_config<true, false, KM_BF16>(config, a, a_scale, b, b_scale, nullptr, nullptr, bias, c, (int)M, (int)N, (int)K, 0, st);
   }
-  if (km) return dispatch_config<true, true, KM_F16>(config, a, a_scale, b, b_scale, nullptr, nullptr, bias, c, (int)M, (int)N, (int)K, st);
-  return dispatch_config<true, false, KM_F16>(config, a, a_scale, b, b_scale, nullptr, nullptr, bias, c, (int)M, (int)N, (int)K, st);
+  if (km) return dispatch_config<true, true, KM_F16>(config, a, a_scale, b, b_scale, nullptr, nullptr, bias, c, (int)M, (int)N, (int)K, 0, st);
+  return dispatch_config<true, false, KM_F16>(config, a, a_scale, b, b_scale, nullptr, nullptr, bias, c, (int)M, (int)N, (int)K, 0, st);
 }
 
 extern "C" int km_gemm_fp8_tensor(const void* a, const float* sa, const void* b, const float* sb,
@@ -460,6 +468,20 @@ extern "C" int km_gemm_fp8_tensor(const void* a, const float* sa, const void* b,
   if (!sa || !sb) return km_fail(KM_ERR_ARG, "km_gemm_fp8_tensor: null scale pointer");
   hipStream_t st = (hipStream_t)stream;
   if (out_dtype == KM_BF16)
-    return dispatch_config<false, false, KM_BF16>(config, a, nullptr, b, nullptr, sa, sb, bias, c, (int)M, (int)N, (int)K, st);
-  return dispatch_config<false, false, KM_F16>(config, a, nullptr, b, nullptr, sa, sb, bias, c, (int)M, (int)N, (int)K, st);
+    return dispatch_config<false, false, KM_BF16>(config, a, nullptr, b, nullptr, sa, sb, bias, c, (int)M, (int)N, (int)K, 0, st);
+  return dispatch_config<false, false, KM_F16>(config, a, nullptr, b, nullptr, sa, sb, bias, c, (int)M, (int)N, (int)K, 0, st);
+}
+
+extern "C" int km_gemm_fp8_rows(const void* a, const float* sa, const void* b, const float* sb,
+                                const void* bias, void* c, int64_t M, int64_t N, int64_t K,
+                                int out_dtype, int config, void* stream) {
+  int rc = check_gemm_args("km_gemm_fp8_rows", a, b, c, M, N, K, out_dtype, config);
+  if (rc != KM_OK) return rc;
+  if (M == 0 || N == 0) return KM_OK;
+  if (!sa || !sb) return km_fail(KM_ERR_ARG, "km_gemm_fp8_rows: null scale pointer");
+  if (reinterpret_cast<uintptr_t>(sb) & 15) return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_fp8_rows: the column scales must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == KM_BF16)
+    return dispatch_config<false, false, KM_BF16>(config, a, nullptr, b, nullptr, sa, sb, bias, c, (int)M, (int)N, (int)K, 1, st);
+  return dispatch_config<false, false, KM_F16>(config, a, nullptr, b, nullptr, sa, sb, bias, c, (int)M, (int)N, (int)K, 1, st);
 }

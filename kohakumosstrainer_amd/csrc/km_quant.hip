@@ -9,6 +9,8 @@
 //   quant_mx_generic  any strides, one thread per block of 32
 //   tensor_amax / tensor_cast   per-tensor recipe (reference formats.py:77-79,
 //                     Triton quantize.py:86-91,161-168)
+//   quant_fp8_rows    per-row recipe, one fp32 scale per row (reference formats.py:80-82,
+//                     Triton quantize.py:64-84,151-158)
 //
 // All of them read each input element once and write each output byte once.
 #include <hip/hip_runtime.h>
@@ -400,6 +402,139 @@ __global__ __launch_bounds__(256) void tensor_cast(const uint16_t* __restrict__ 
   }
 }
 
+// ---- per-row recipe ----------------------------------------------------------------------------
+// s[r] = max(amax_r, 1e-12) / 448 and q = e4m3(clamp(x / s[r])), both IEEE fp32 divisions
+// (reference formats.py:80-82, Triton quantize.py:64-84). One wavefront per row.
+__device__ __forceinline__ uint32_t wave_max(uint32_t m) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const uint32_t o = (uint32_t)__shfl_xor((int)m, off);
+    m = o > m ? o : m;
+  }
+  return m;
+}
+
+// Codes of a row whose amax is infinite or NaN, where clamp-and-convert instructions and the
+// reference's host arithmetic part ways. Scale inf: finite x / inf is a signed zero, inf / inf
+// is NaN. Scale NaN: every quotient is NaN; the reference's host division hands back the
+// scale's NaN (code 0x7F) unless x is a NaN itself (code 0xFF, as for inf / inf).
+template <int DT>
+__device__ __forceinline__ uint32_t nonfinite_row_code(uint32_t h, bool nan_row) {
+  const uint32_t a = h & 0x7FFFu;
+  if (nan_row) return a > inf16<DT>() ? 0xFFu : 0x7Fu;
+  return a == inf16<DT>() ? 0xFFu : (h >> 8) & 0x80u;
+}
+
+template <int DT>
+__device__ __forceinline__ uint2 row_codes8(const uint4& raw, float s, bool finite, bool nan_row) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  uint32_t out[2];
+  if (finite) {
+    float f[8];
+    widen8<DT>(raw, f);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = __builtin_amdgcn_fmed3f(__fdiv_rn(f[i], s), -448.0f, 448.0f);
+    out[0] = cvt4_f32(f[0], f[1], f[2], f[3], 1.0f);
+    out[1] = cvt4_f32(f[4], f[5], f[6], f[7], 1.0f);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      out[i] = nonfinite_row_code<DT>(w[2 * i] & 0xFFFFu, nan_row) | (nonfinite_row_code<DT>(w[2 * i] >> 16, nan_row) << 8) |
+               (nonfinite_row_code<DT>(w[2 * i + 1] & 0xFFFFu, nan_row) << 16) | (nonfinite_row_code<DT>(w[2 * i + 1] >> 16, nan_row) << 24);
+    }
+  }
+  return make_uint2(out[0], out[1]);
+}
+
+// scale of a row from the largest 16-bit absolute-value pattern in it
+template <int DT>
+__device__ __forceinline__ float row_scale_of(uint32_t m16) {
+  if (m16 > inf16<DT>()) return bits_f32(0x7FC00000u);
+  const uint32_t ab = widen_bits<DT>(m16);
+  return __fdiv_rn(bits_f32(ab > kAmaxFloorBits ? ab : kAmaxFloorBits), 448.0f);
+}
+
+constexpr int kRowRecipeHeld = 8;  // 128-bit loads a lane keeps in registers: rows up to 4096 elements are read once
+
+// Unit-stride rows, cols = 8 * chunks. HELD: the whole row stays in registers between the
+// amax pass and the conversion; otherwise the second pass reads it again (from L2: a wavefront
+// re-reads what it has just fetched).
+template <int DT, bool HELD>
+__global__ __launch_bounds__(256) void quant_fp8_rows(const uint16_t* __restrict__ x, int64_t ld, uint32_t chunks,
+                                                      uint32_t rows, uint8_t* __restrict__ q, float* __restrict__ scale) {
+  saturating_conversions();
+  const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const uint32_t lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const uint4* src = reinterpret_cast<const uint4*>(x + (uint64_t)row * (uint64_t)ld);
+  uint2* dst = reinterpret_cast<uint2*>(q + (uint64_t)row * chunks * 8);
+  uint4 raw[HELD ? kRowRecipeHeld : 1];
+  uint32_t m16 = 0;
+  if constexpr (HELD) {
+#pragma unroll
+    for (int u = 0; u < kRowRecipeHeld; ++u) {
+      const uint32_t c = lane + 64 * u;
+      raw[u] = c < chunks ? src[c] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < kRowRecipeHeld; ++u) {
+      const uint32_t a = amax16x8(raw[u]);
+      m16 = a > m16 ? a : m16;
+    }
+  } else {
+    for (uint32_t c = lane; c < chunks; c += 64) {
+      const uint32_t a = amax16x8(src[c]);
+      m16 = a > m16 ? a : m16;
+    }
+  }
+  m16 = wave_max(m16);
+  const float s = row_scale_of<DT>(m16);
+  if (lane == 0) scale[row] = s;
+  const bool finite = m16 < inf16<DT>(), nan_row = m16 > inf16<DT>();
+  if constexpr (HELD) {
+#pragma unroll
+    for (int u = 0; u < kRowRecipeHeld; ++u) {
+      const uint32_t c = lane + 64 * u;
+      if (c < chunks) dst[c] = row_codes8<DT>(raw[u], s, finite, nan_row);
+    }
+  } else {
+    for (uint32_t c = lane; c < chunks; c += 64) dst[c] = row_codes8<DT>(src[c], s, finite, nan_row);
+  }
+}
+
+// Any strides and lengths: one wavefront per row, one element per lane and trip.
+template <int DT>
+__global__ __launch_bounds__(256) void quant_fp8_rows_generic(const uint16_t* __restrict__ x, int64_t sr, int64_t sc,
+                                                              uint32_t rows, int64_t cols, uint8_t* __restrict__ q,
+                                                              float* __restrict__ scale) {
+  saturating_conversions();
+  const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const uint32_t lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const uint16_t* src = x + (int64_t)row * sr;
+  uint32_t m16 = 0;
+  for (int64_t c = lane; c < cols; c += 64) {
+    const uint32_t a = src[c * sc] & 0x7FFFu;
+    m16 = a > m16 ? a : m16;
+  }
+  m16 = wave_max(m16);
+  const float s = row_scale_of<DT>(m16);
+  if (lane == 0) scale[row] = s;
+  const bool finite = m16 < inf16<DT>(), nan_row = m16 > inf16<DT>();
+  uint8_t* dst = q + (int64_t)row * cols;
+  for (int64_t c = lane; c < cols; c += 64) {
+    const uint32_t h = src[c * sc];
+    uint32_t code;
+    if (finite) {
+      const float d = __builtin_amdgcn_fmed3f(__fdiv_rn(widen<DT>(h), s), -448.0f, 448.0f);
+      code = cvt4_f32(d, 0.f, 0.f, 0.f, 1.0f) & 0xFFu;
+    } else {
+      code = nonfinite_row_code<DT>(h, nan_row);
+    }
+    dst[c] = (uint8_t)code;
+  }
+}
+
 }  // namespace km
 
 using namespace km;
@@ -490,4 +625,30 @@ extern "C" int km_quant_tensor(const void* x, int64_t rows, int64_t cols, int64_
     hipLaunchKernelGGL(tensor_cast<DT>, dim3(blocks), dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, amax_workspace, (uint8_t*)q, scale_out);
   });
   return km_check_launch("km_quant_tensor");
+}
+
+extern "C" int km_quant_rows(const void* x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,
+                             int dtype, void* q, float* scale_out, void* stream) {
+  if (dtype != KM_BF16 && dtype != KM_F16) return km_fail(KM_ERR_ARG, "km_quant_rows: dtype must be bf16 or f16");
+  if (rows < 0 || cols < 0) return km_fail(KM_ERR_ARG, "km_quant_rows: negative shape");
+  if (rows == 0) return KM_OK;
+  if (rows > 0x7FFFFFFFll) return km_fail(KM_ERR_ARG, "km_quant_rows: too many rows");
+  if (!scale_out || (cols > 0 && (!x || !q))) return km_fail(KM_ERR_ARG, "km_quant_rows: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const uint16_t* xp = (const uint16_t*)x;
+  const dim3 grid((unsigned)((rows + 3) / 4));
+  const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0;
+  if (stride_col == 1 && aligned && cols % 8 == 0 && stride_row % 8 == 0 && stride_row >= cols && cols / 8 <= 0x7FFFFFFFll) {
+    const uint32_t chunks = (uint32_t)(cols / 8);
+    KM_DISPATCH_DT(dtype, {
+      if (chunks <= 64u * kRowRecipeHeld)
+        hipLaunchKernelGGL((quant_fp8_rows<DT, true>), grid, dim3(256), 0, st, xp, stride_row, chunks, (uint32_t)rows, (uint8_t*)q, scale_out);
+      else
+        hipLaunchKernelGGL((quant_fp8_rows<DT, false>), grid, dim3(256), 0, st, xp, stride_row, chunks, (uint32_t)rows, (uint8_t*)q, scale_out);
+    });
+  } else {
+    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL(quant_fp8_rows_generic<DT>, grid, dim3(256), 0, st, xp, stride_row, stride_col,
+                                             (uint32_t)rows, cols, (uint8_t*)q, scale_out));
+  }
+  return km_check_launch("km_quant_rows");
 }

@@ -5,9 +5,10 @@ quantizer. Host-side counterpart of reference `backends/triton/fp8/linear.py` (c
 :88-118, runner :162-196, `_select` :254-286, launchers :289-301, registration :309-320).
 
 Recipes served on the GPU: `mx` (block-scaled MFMA; the activation quantizer writes the
-MFMA-packed scales directly, the weight's packed copy comes in `aux` or is packed per call)
-and `tensor` (plain fp8 MFMA, scalar scales on the accumulator). `row` and `block` are not
-built yet and are refused by the support check. The 16-bit input gradient of a base stored
+MFMA-packed scales directly, the weight's packed copy comes in `aux` or is packed per call),
+`tensor` (plain fp8 MFMA, scalar scales on the accumulator) and `row` (the same GEMM with one
+scale per output row and one per output column on the accumulator). `block` is not built yet
+and is refused by the support check. The 16-bit input gradient of a base stored
 without a dgrad copy is `dy @ dequantize(W)`: an elementwise dequantize and a plain library
 GEMM, as in the reference's `w16` path.
 """
@@ -23,7 +24,7 @@ from kohakumosstrainer_amd.kernels.fp8.op import make_fp8_linear, make_fp8_linea
 from kohakumosstrainer_amd.kernels.fp8.train import make_fp8_linear_train
 from kohakumosstrainer_amd.kernels.tuning import pow2
 
-GPU_RECIPES = ("mx", "tensor")
+GPU_RECIPES = ("mx", "tensor", "row")
 ALIGN_K = 128
 _RESOLVED: dict[tuple, dict] = {}
 tuning.on_reset(_RESOLVED.clear)
@@ -57,6 +58,9 @@ def _run(cfg, recipe, a, bq, bs, baux, bias):
         if baux is None or baux.numel() != packed_numel(bq.shape[0], bq.shape[1]) or baux.dtype != torch.uint8:
             baux = native.pack_scales(bs)
         return native.gemm_mx(aq, a_packed, bq, baux, bias, a.dtype, cfg["id"], packed=True)
+    if recipe == "row":
+        aq, sa = native.quant_rows(a)
+        return native.gemm_fp8_rows(aq, sa, bq, bs.float(), bias, a.dtype, cfg["id"])
     aq, sa = native.quant_tensor(a)
     return native.gemm_fp8_tensor(aq, sa, bq, bs.reshape(1).float(), bias, a.dtype, cfg["id"])
 

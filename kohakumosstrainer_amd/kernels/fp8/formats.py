@@ -9,8 +9,8 @@ An operand is 2-D `[rows, K]` with K the contraction axis; codes are e4m3fn (max
 
 Interface and arithmetic follow reference `src/kohakumoss_kernels/fp8/formats.py:70-136`.
 `quantize` runs the hand-written HIP quantizers for device tensors of the recipes the GPU
-path serves (mx, tensor; bf16 / fp16 input) and plain torch ops otherwise (host tensors, the
-row and block recipes, fp32 input): both produce the same bytes. `pack_mx` builds the
+path serves (mx, tensor, row; bf16 / fp16 input) and plain torch ops otherwise (host tensors,
+the block recipe, fp32 input): both produce the same bytes. `pack_mx` builds the
 MFMA-packed scale copy the HIP GEMM reads (the role `swizzle_mx` plays for a vendor GEMM).
 """
 
@@ -87,11 +87,11 @@ def quantize(x: Tensor, recipe: str, role: str = "act") -> tuple[Tensor, Tensor]
     """`(q e4m3 [rows, K], scale)` of a 2-D operand under `recipe`; `role` matters only for
     `block` (weights scale 128x128 blocks)."""
     _check(x, recipe, role)
-    if x.device.type == "cuda" and x.dtype in _HIP_DTYPES and recipe in ("mx", "tensor") and x.numel():
+    if x.device.type == "cuda" and x.dtype in _HIP_DTYPES and recipe in ("mx", "tensor", "row") and x.numel():
         from kohakumosstrainer_amd import native
 
         x = x.detach()
-        return native.quant_mx(x) if recipe == "mx" else native.quant_tensor(x)
+        return {"mx": native.quant_mx, "tensor": native.quant_tensor, "row": native.quant_rows}[recipe](x)
     return _quantize_torch(x, recipe, role)
 
 

@@ -30,8 +30,10 @@ EXPORTS = (
     "km_scales_packed_bytes",
     "km_scales_pack",
     "km_quant_tensor",
+    "km_quant_rows",
     "km_gemm_mx",
     "km_gemm_fp8_tensor",
+    "km_gemm_fp8_rows",
     "km_wo_gemm_fwd",
     "km_wo_gemm_dgrad",
     "km_num_configs",
@@ -59,8 +61,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.km_scales_packed_bytes.argtypes = [i64, i64]
     lib.km_scales_pack.argtypes = [p, i64, i64, p, p]
     lib.km_quant_tensor.argtypes = [p, i64, i64, i64, i64, i32, p, p, p, p]
+    lib.km_quant_rows.argtypes = [p, i64, i64, i64, i64, i32, p, p, p]
     lib.km_gemm_mx.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_gemm_fp8_tensor.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
+    lib.km_gemm_fp8_rows.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_wo_gemm_fwd.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_wo_gemm_dgrad.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_num_configs.argtypes = [i32]
@@ -203,6 +207,19 @@ def quant_tensor(x: Tensor) -> tuple[Tensor, Tensor]:
     return q.view(E4M3), s
 
 
+def quant_rows(x: Tensor) -> tuple[Tensor, Tensor]:
+    """`(q e4m3 [rows, K], scale fp32 [rows])` under the per-row recipe; any strides."""
+    if x.dim() != 2:
+        raise ValueError(f"fp8 operand must be 2-D, got {tuple(x.shape)}")
+    _on_gpu(x)
+    rows, k = x.shape
+    q = torch.empty(rows, k, device=x.device, dtype=torch.uint8)
+    s = torch.empty(rows, device=x.device, dtype=torch.float32)
+    with torch.cuda.device(x.device):
+        _check(load().km_quant_rows(x.data_ptr(), rows, k, x.stride(0), x.stride(1), _dtype_code(x.dtype), q.data_ptr(), s.data_ptr(), _stream(x)))
+    return q.view(E4M3), s
+
+
 # ---- GEMMs --------------------------------------------------------------------------------
 
 
@@ -258,6 +275,18 @@ def gemm_fp8_tensor(a: Tensor, sa: Tensor, b: Tensor, sb: Tensor, bias: Tensor |
     _on_gpu(a, sa, sb)
     with torch.cuda.device(a.device):
         _check(load().km_gemm_fp8_tensor(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), None if bias is None else bias.data_ptr(), c.data_ptr(), m, n, k, _dtype_code(out_dtype), config, _stream(a)))
+    return c
+
+
+def gemm_fp8_rows(a: Tensor, sa: Tensor, b: Tensor, sb: Tensor, bias: Tensor | None, out_dtype: torch.dtype, config: int = 0) -> Tensor:
+    """`(a b^T) * sa[:, None] * sb[None, :] + bias`, sa `[M]` and sb `[N]` fp32 device vectors."""
+    a, b, bias, c, m, n, k = _gemm_operands(a, b, bias, out_dtype)
+    if tuple(sa.shape) != (m,) or tuple(sb.shape) != (n,) or sa.dtype != torch.float32 or sb.dtype != torch.float32:
+        raise ValueError(f"per-row scales must be fp32 vectors [{m}] and [{n}], got {tuple(sa.shape)} {sa.dtype} and {tuple(sb.shape)} {sb.dtype}")
+    _on_gpu(a, sa, sb)
+    sa, sb = sa.contiguous(), sb.contiguous()
+    with torch.cuda.device(a.device):
+        _check(load().km_gemm_fp8_rows(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), None if bias is None else bias.data_ptr(), c.data_ptr(), m, n, k, _dtype_code(out_dtype), config, _stream(a)))
     return c
 
 

@@ -1,4 +1,4 @@
-"""HIP fp8 GEMMs (block-scaled MXFP8 and per-tensor) through the C ABI against the fp64
+"""HIP fp8 GEMMs (block-scaled MXFP8, per-tensor and per-row) through the C ABI against the fp64
 product of the exactly dequantized operands, next to the oracle's eager result, with
 the reference's pass rule (`oracle.stats.assert_no_regression`, 10x rule; reference
 `tests/kernels/quant/test_fp8.py:117-148`, `test_fp8_accumulation.py:83-90`).
@@ -126,6 +126,30 @@ def test_tensor_gemm(dtype, m, n, k):
         y = native.gemm_fp8_tensor(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), bias.cuda(), dtype, cfg)
         assert_no_regression(y.cpu(), eager, truth, f"tensor cfg{cfg} {m}x{n}x{k}")
         assert rel_l2(y.cpu(), truth) <= (REL_L2_BF16 if dtype == torch.bfloat16 else REL_L2_F16)
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+@pytest.mark.parametrize("m,n,k", [(200, 384, 256), (1000, 512, 384), (1, 128, 128), (513, 200, 256)])
+def test_row_gemm(dtype, m, n, k):
+    """Row recipe: per-row activation scales and per-row weight scales on the accumulator. Rows
+    of very different magnitude make a swapped or scalar scale visible."""
+    x, w, bias = operands(m, n, k, dtype, seed=4, x_scale=torch.logspace(-2, 2, m)[:, None])
+    w = w * torch.logspace(-1, 1, n)[:, None]
+    xq, xs = formats.quantize(x, "row")
+    wq, ws = formats.quantize(w, "row", "weight")
+    truth = linear.exact64(xq, xs, "row") @ linear.exact64(wq, ws, "row").T + bias.double()
+    eager = linear.fp8_forward(x, wq, ws, None, bias, "row")
+    for cfg in range(n_configs()):
+        y = native.gemm_fp8_rows(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), bias.cuda(), dtype, cfg)
+        assert_no_regression(y.cpu(), eager, truth, f"row cfg{cfg} {m}x{n}x{k}")
+        assert rel_l2(y.cpu(), truth) <= (REL_L2_BF16 if dtype == torch.bfloat16 else REL_L2_F16)
+    if m > 1:
+        bad = native.gemm_fp8_rows(xq.cuda(), xs.flip(0).cuda(), wq.cuda(), ws.cuda(), bias.cuda(), dtype, 0).cpu()
+        must_fail(lambda: assert_no_regression(bad, eager, truth, "flipped"), "activation scales in the wrong row order")
+        bad = native.gemm_fp8_rows(xq.cuda(), xs.cuda(), wq.cuda(), ws.roll(1).cuda(), bias.cuda(), dtype, 0).cpu()
+        must_fail(lambda: assert_no_regression(bad, eager, truth, "rolled"), "weight scales on the wrong column")
+    with pytest.raises(ValueError):
+        native.gemm_fp8_rows(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda()[:1], None, dtype, 0)
 
 
 def test_gemm_argument_errors():

@@ -65,7 +65,7 @@ def check(got, eager, exact, dtype, what, slack=1.0):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("recipe,dgrad", [("mx", True), ("mx", False), ("tensor", True)])
+@pytest.mark.parametrize("recipe,dgrad", [("mx", True), ("mx", False), ("tensor", True), ("row", True), ("row", False)])
 def test_fp8_linear_forward_and_grads(dtype, recipe, dgrad):
     m, n, k = 300, 384, 512
     x, w, bias, dy, base = problem(m, n, k, dtype, recipe, dgrad)
@@ -86,7 +86,10 @@ def test_fp8_linear_forward_and_grads(dtype, recipe, dgrad):
         exact_dx = exact_product(dy, base.q_t, base.scale_t, None, recipe)
     else:
         exact_dx = dy.double() @ oracle_linear.exact64(base.q, base.scale, recipe)
-    check(xd.grad, eager_dx, exact_dx, dtype, f"dgrad {recipe} fp8={dgrad}")
+    # the 16-bit path rounds q * scale to the activation dtype first: exact for mx (powers of
+    # two), one more 2^-9 rounding per weight for fp32 scales, in the eager path just the same
+    slack = 1.0 if dgrad or recipe == "mx" else 2.0
+    check(xd.grad, eager_dx, exact_dx, dtype, f"dgrad {recipe} fp8={dgrad}", slack)
     assert torch.equal(bd.grad.cpu(), oracle_linear.bias_grad(dy, dtype))
 
 

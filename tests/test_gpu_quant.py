@@ -1,5 +1,5 @@
 """HIP quantizers against the CPU oracle, bit for bit, through the C ABI
-(`native.quant_mx` / `native.quant_tensor`). Mirrors reference
+(`native.quant_mx` / `native.quant_tensor` / `native.quant_rows`). Mirrors reference
 `tests/kernels/quant/test_fp8.py:61-82` (bytes equal the eager reference, strided input)
 and adds the column-wise (transposed) case, an exhaustive bf16 sweep and the full-size
 `[16384, 3072]` operand with outliers."""
@@ -166,6 +166,83 @@ def test_tensor_recipe_all_zero_and_weight_like():
     q, s = native.quant_tensor(w.cuda())
     rq, rs = formats.quantize(w, "tensor")
     assert torch.equal(s.cpu(), rs) and torch.equal(u8(q).cpu(), u8(rq))
+
+
+def check_rows(x_cpu: torch.Tensor, view=lambda t: t):
+    q, s = native.quant_rows(view(x_cpu.cuda()))
+    rq, rs = formats.quantize(view(x_cpu), "row")
+    assert q.dtype == torch.float8_e4m3fn and s.dtype == torch.float32 and s.shape == (rq.shape[0],)
+    assert q.shape == rq.shape and q.is_contiguous()
+    assert torch.equal(s.cpu().view(torch.int32), rs.view(torch.int32)), "scale bits"
+    assert torch.equal(u8(q).cpu(), u8(rq)), "code bytes"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,k", [(300, 1024), (5, 7), (1, 1), (64, 200), (33, 4096), (9, 4104), (130, 8192), (3, 12288)])
+def test_row_recipe_bytes_equal_oracle(dtype, m, k):
+    """Reference `tests/kernels/quant/test_fp8.py:61-82` for the row recipe: rows kept in
+    registers (K <= 4096), rows read twice (K > 4096), ragged K (element-wise kernel) and the
+    transposed view `quantize(w.t(), "row")` of the input-gradient weight copy."""
+    x = activations(m, k, dtype, seed=11)
+    check_rows(x)
+    check_rows(x, view=lambda t: t.t())
+    if k >= 16:
+        check_rows(x, view=lambda t: t[:, 8:])          # unit stride, rows not densely packed
+        check_rows(x, view=lambda t: t[:, 1 : k - 1])   # not 16-byte aligned
+
+
+def test_row_recipe_power_of_two_scales_hit_rounding_ties():
+    """With amax = 448 * 2^e the scale is 2^e and x / s is exact, so bf16 inputs (8 significand
+    bits) land on e4m3 ties (4 significand bits), in its subnormal range and on the clamp."""
+    bits = torch.arange(0x3000, 0x4400, dtype=torch.int32)  # every bf16 pattern in [2^-31, 512)
+    vals = (bits << 16).view(torch.float32)
+    rows = []
+    for e in (-20, -3, 0, 5, 40):
+        r = vals * 2.0**e
+        r = torch.where(r.abs() > 448 * 2.0**e, torch.zeros(()), r)
+        r[0] = 448 * 2.0**e
+        rows += [r, -r]
+    x = torch.stack(rows).to(torch.bfloat16)
+    assert torch.equal(x.float(), torch.stack(rows))
+    check_rows(x)                                   # 5120 columns: the re-reading kernel
+    check_rows(x[:, :4096].contiguous())            # rows held in registers
+    check_rows(x.to(torch.float16)[4:8])
+
+
+def test_row_recipe_zero_tiny_inf_and_nan_rows():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(8, 256, generator=g)
+    x[0] = 0.0
+    x[1] = 1e-20                                   # below the 1e-12 amax floor
+    x[2, 5] = float("inf")
+    x[2, 6] = float("-inf")
+    x[3, 7] = float("nan")
+    x[4, ::2] = -0.0
+    x[5] *= 1e30
+    x[6] *= 1e-30
+    x = x.to(torch.bfloat16)
+    q, s = native.quant_rows(x.cuda())
+    rq, rs = formats.quantize(x, "row")
+    assert torch.equal(torch.isnan(s.cpu()), torch.isnan(rs))
+    keep = ~torch.isnan(rs)
+    assert torch.equal(s.cpu()[keep].view(torch.int32), rs[keep].view(torch.int32))
+    assert torch.equal(u8(q).cpu(), u8(rq))
+    assert s.cpu()[0].item() == rs[0].item() == torch.tensor(1e-12).div(torch.tensor(448.0)).item()
+
+
+def test_row_recipe_full_size_activation():
+    x = outlier_operand()
+    check_rows(x)
+
+
+def test_row_recipe_argument_errors():
+    x = torch.zeros(4, 8, device="cuda")
+    with pytest.raises(ValueError):
+        native.quant_rows(x)  # fp32 input
+    with pytest.raises(ValueError):
+        native.quant_rows(x.bfloat16()[0])
+    q, s = native.quant_rows(x.bfloat16()[:0])
+    assert q.shape == (0, 8) and s.shape == (0,)
 
 
 def test_mx_committed_vectors_rows_and_cols():
