@@ -56,26 +56,6 @@ __device__ __forceinline__ void widen8(const uint4& raw, float (&f)[8]) {
   }
 }
 
-__device__ __forceinline__ uint32_t amax_bits8(const float (&f)[8]) {
-  uint32_t m = 0;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    uint32_t a = f32_bits(f[i]) & kAbsMask;
-    m = a > m ? a : m;
-  }
-  return m;
-}
-
-__device__ __forceinline__ uint2 encode8(const float (&f)[8], float inv) {
-  uint32_t lo = 0, hi = 0;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    lo |= e4m3_encode(f[i] * inv) << (8 * i);
-    hi |= e4m3_encode(f[4 + i] * inv) << (8 * i);
-  }
-  return make_uint2(lo, hi);
-}
-
 // ---- hardware e4m3 conversion ----------------------------------------------------------------
 // V_CVT_SCALEF32_PK_FP8_{BF16,F16,F32} divide by the power of two in the exponent field of the
 // scale operand, round once to nearest even and, with MODE.FP16_OVFL set, saturate at +-448: the
@@ -334,77 +314,9 @@ __global__ __launch_bounds__(256) void scales_pack(const uint8_t* __restrict__ i
   out[scale_pack_offset(r, b, (rows + 127) >> 7)] = in[i];
 }
 
-// ---- per-tensor recipe -----------------------------------------------------------------------
-__global__ void fill_u32(uint32_t* p, uint32_t v) { *p = v; }
-
-template <int DT>
-__global__ __launch_bounds__(256) void tensor_amax(const uint16_t* __restrict__ x, int64_t sr,
-                                                   int64_t sc, int64_t rows, int64_t cols,
-                                                   uint32_t* __restrict__ amax_bits) {
-  // non-negative floats order like their bits: an unsigned atomic max is an abs-max
-  const int64_t n = rows * cols;
-  const bool dense = sc == 1 && sr == cols;
-  uint32_t m = 0;
-  const int64_t stride = (int64_t)gridDim.x * 256;
-  if (dense && (cols % 8) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
-    for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < n / 8; g += stride) {
-      float f[8];
-      widen8<DT>(reinterpret_cast<const uint4*>(x)[g], f);
-      const uint32_t a = amax_bits8(f);
-      m = a > m ? a : m;
-    }
-  } else {
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
-      const int64_t r = i / cols, c = i - r * cols;
-      const uint32_t a = f32_bits(widen<DT>(x[r * sr + c * sc])) & kAbsMask;
-      m = a > m ? a : m;
-    }
-  }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    const uint32_t o = (uint32_t)__shfl_xor((int)m, off);
-    m = o > m ? o : m;
-  }
-  if ((threadIdx.x & 63) == 0 && m != 0) atomicMax(amax_bits, m);
-}
-
-// s = max(amax, 1e-12) / 448 and q = e4m3(clamp(x / s)), both IEEE fp32 divisions.
-template <int DT>
-__global__ __launch_bounds__(256) void tensor_cast(const uint16_t* __restrict__ x, int64_t sr,
-                                                   int64_t sc, int64_t rows, int64_t cols,
-                                                   const uint32_t* __restrict__ amax_bits,
-                                                   uint8_t* __restrict__ q,
-                                                   float* __restrict__ scale_out) {
-  uint32_t ab = *amax_bits;
-  ab = ab > kAmaxFloorBits ? ab : kAmaxFloorBits;
-  const float s = __fdiv_rn(bits_f32(ab), 448.0f);
-  if (blockIdx.x == 0 && threadIdx.x == 0 && scale_out) *scale_out = s;
-  const int64_t n = rows * cols;
-  const bool dense = sc == 1 && sr == cols;
-  const int64_t stride = (int64_t)gridDim.x * 256;
-  if (dense && (cols % 8) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
-    for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < n / 8; g += stride) {
-      float f[8];
-      widen8<DT>(reinterpret_cast<const uint4*>(x)[g], f);
-      uint32_t lo = 0, hi = 0;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        lo |= e4m3_encode(__fdiv_rn(f[i], s)) << (8 * i);
-        hi |= e4m3_encode(__fdiv_rn(f[4 + i], s)) << (8 * i);
-      }
-      reinterpret_cast<uint2*>(q)[g] = make_uint2(lo, hi);
-    }
-  } else {
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
-      const int64_t r = i / cols, c = i - r * cols;
-      q[i] = (uint8_t)e4m3_encode(__fdiv_rn(widen<DT>(x[r * sr + c * sc]), s));
-    }
-  }
-}
-
-// ---- per-row recipe ----------------------------------------------------------------------------
-// s[r] = max(amax_r, 1e-12) / 448 and q = e4m3(clamp(x / s[r])), both IEEE fp32 divisions
-// (reference formats.py:80-82, Triton quantize.py:64-84). One wavefront per row.
+// ---- fp32-scale recipes (per row, per tensor) ---------------------------------------------------
+// s = max(amax, 1e-12) / 448 and q = e4m3(clamp(x / s)), both IEEE fp32 divisions (reference
+// formats.py:41-45).
 __device__ __forceinline__ uint32_t wave_max(uint32_t m) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
@@ -414,19 +326,19 @@ __device__ __forceinline__ uint32_t wave_max(uint32_t m) {
   return m;
 }
 
-// Codes of a row whose amax is infinite or NaN, where clamp-and-convert instructions and the
+// Codes of a row (tensor) whose amax is infinite or NaN, where clamp-and-convert instructions and the
 // reference's host arithmetic part ways. Scale inf: finite x / inf is a signed zero, inf / inf
 // is NaN. Scale NaN: every quotient is NaN; the reference's host division hands back the
 // scale's NaN (code 0x7F) unless x is a NaN itself (code 0xFF, as for inf / inf).
 template <int DT>
-__device__ __forceinline__ uint32_t nonfinite_row_code(uint32_t h, bool nan_row) {
+__device__ __forceinline__ uint32_t nonfinite_code(uint32_t h, bool nan_row) {
   const uint32_t a = h & 0x7FFFu;
   if (nan_row) return a > inf16<DT>() ? 0xFFu : 0x7Fu;
   return a == inf16<DT>() ? 0xFFu : (h >> 8) & 0x80u;
 }
 
 template <int DT>
-__device__ __forceinline__ uint2 row_codes8(const uint4& raw, float s, bool finite, bool nan_row) {
+__device__ __forceinline__ uint2 divided_codes8(const uint4& raw, float s, bool finite, bool nan_row) {
   const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
   uint32_t out[2];
   if (finite) {
@@ -439,21 +351,111 @@ __device__ __forceinline__ uint2 row_codes8(const uint4& raw, float s, bool fini
   } else {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      out[i] = nonfinite_row_code<DT>(w[2 * i] & 0xFFFFu, nan_row) | (nonfinite_row_code<DT>(w[2 * i] >> 16, nan_row) << 8) |
-               (nonfinite_row_code<DT>(w[2 * i + 1] & 0xFFFFu, nan_row) << 16) | (nonfinite_row_code<DT>(w[2 * i + 1] >> 16, nan_row) << 24);
+      out[i] = nonfinite_code<DT>(w[2 * i] & 0xFFFFu, nan_row) | (nonfinite_code<DT>(w[2 * i] >> 16, nan_row) << 8) |
+               (nonfinite_code<DT>(w[2 * i + 1] & 0xFFFFu, nan_row) << 16) | (nonfinite_code<DT>(w[2 * i + 1] >> 16, nan_row) << 24);
     }
   }
   return make_uint2(out[0], out[1]);
 }
 
-// scale of a row from the largest 16-bit absolute-value pattern in it
 template <int DT>
-__device__ __forceinline__ float row_scale_of(uint32_t m16) {
+__device__ __forceinline__ uint32_t divided_code1(uint32_t h, float s, bool finite, bool nan_row) {
+  if (!finite) return nonfinite_code<DT>(h, nan_row);
+  const float d = __builtin_amdgcn_fmed3f(__fdiv_rn(widen<DT>(h), s), -448.0f, 448.0f);
+  return cvt4_f32(d, 0.f, 0.f, 0.f, 1.0f) & 0xFFu;
+}
+
+// scale from the largest 16-bit absolute-value pattern of a row
+template <int DT>
+__device__ __forceinline__ float scale_of_amax16(uint32_t m16) {
   if (m16 > inf16<DT>()) return bits_f32(0x7FC00000u);
   const uint32_t ab = widen_bits<DT>(m16);
   return __fdiv_rn(bits_f32(ab > kAmaxFloorBits ? ab : kAmaxFloorBits), 448.0f);
 }
 
+// ---- per-tensor recipe -----------------------------------------------------------------------
+__global__ void fill_u32(uint32_t* p, uint32_t v) { *p = v; }
+
+constexpr int kTensorBlocks = 2048;  // grid-stride: 8 workgroups per compute unit, one atomic each
+
+// non-negative floats order like their bits: an unsigned atomic max of fp32 bits is an abs-max
+// (NaN patterns stay above infinity)
+template <int DT>
+__global__ __launch_bounds__(256) void tensor_amax(const uint16_t* __restrict__ x, int64_t sr,
+                                                   int64_t sc, int64_t rows, int64_t cols,
+                                                   uint32_t* __restrict__ amax_bits) {
+  const int64_t n = rows * cols;
+  const bool dense = sc == 1 && sr == cols;
+  uint32_t m16 = 0;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  if (dense && (cols % 8) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    const uint4* src = reinterpret_cast<const uint4*>(x);
+    const int64_t nch = n / 8;
+    int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    for (; g + 3 * stride < nch; g += 4 * stride) {
+      const uint4 r0 = src[g], r1 = src[g + stride], r2 = src[g + 2 * stride], r3 = src[g + 3 * stride];
+      const uint32_t a = amax16x8(r0), b = amax16x8(r1), c = amax16x8(r2), d = amax16x8(r3);
+      const uint32_t ab = a > b ? a : b, cd = c > d ? c : d, abcd = ab > cd ? ab : cd;
+      m16 = abcd > m16 ? abcd : m16;
+    }
+    for (; g < nch; g += stride) {
+      const uint32_t a = amax16x8(src[g]);
+      m16 = a > m16 ? a : m16;
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+      const int64_t r = i / cols, c = i - r * cols;
+      const uint32_t a = x[r * sr + c * sc] & 0x7FFFu;
+      m16 = a > m16 ? a : m16;
+    }
+  }
+  __shared__ uint32_t wave_m[4];
+  const uint32_t m = wave_max(m16);
+  if ((threadIdx.x & 63) == 0) wave_m[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const uint32_t a = wave_m[0] > wave_m[1] ? wave_m[0] : wave_m[1], b = wave_m[2] > wave_m[3] ? wave_m[2] : wave_m[3];
+    const uint32_t bits = widen_bits<DT>(a > b ? a : b);
+    if (bits != 0) atomicMax(amax_bits, bits);
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void tensor_cast(const uint16_t* __restrict__ x, int64_t sr,
+                                                   int64_t sc, int64_t rows, int64_t cols,
+                                                   const uint32_t* __restrict__ amax_bits,
+                                                   uint8_t* __restrict__ q,
+                                                   float* __restrict__ scale_out) {
+  saturating_conversions();
+  const uint32_t ab = *amax_bits;
+  const bool finite = ab < kInfBits, nan_all = ab > kInfBits;
+  const float s = nan_all ? bits_f32(0x7FC00000u) : __fdiv_rn(bits_f32(ab > kAmaxFloorBits ? ab : kAmaxFloorBits), 448.0f);
+  if (blockIdx.x == 0 && threadIdx.x == 0 && scale_out) *scale_out = s;
+  const int64_t n = rows * cols;
+  const bool dense = sc == 1 && sr == cols;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  if (dense && (cols % 8) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    const uint4* src = reinterpret_cast<const uint4*>(x);
+    uint2* dst = reinterpret_cast<uint2*>(q);
+    const int64_t nch = n / 8;
+    int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    for (; g + 3 * stride < nch; g += 4 * stride) {
+      const uint4 r0 = src[g], r1 = src[g + stride], r2 = src[g + 2 * stride], r3 = src[g + 3 * stride];
+      dst[g] = divided_codes8<DT>(r0, s, finite, nan_all);
+      dst[g + stride] = divided_codes8<DT>(r1, s, finite, nan_all);
+      dst[g + 2 * stride] = divided_codes8<DT>(r2, s, finite, nan_all);
+      dst[g + 3 * stride] = divided_codes8<DT>(r3, s, finite, nan_all);
+    }
+    for (; g < nch; g += stride) dst[g] = divided_codes8<DT>(src[g], s, finite, nan_all);
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+      const int64_t r = i / cols, c = i - r * cols;
+      q[i] = (uint8_t)divided_code1<DT>(x[r * sr + c * sc], s, finite, nan_all);
+    }
+  }
+}
+
+// ---- per-row recipe: one wavefront per row -----------------------------------------------------
 constexpr int kRowRecipeHeld = 8;  // 128-bit loads a lane keeps in registers: rows up to 4096 elements are read once
 
 // Unit-stride rows, cols = 8 * chunks. HELD: the whole row stays in registers between the
@@ -488,17 +490,17 @@ __global__ __launch_bounds__(256) void quant_fp8_rows(const uint16_t* __restrict
     }
   }
   m16 = wave_max(m16);
-  const float s = row_scale_of<DT>(m16);
+  const float s = scale_of_amax16<DT>(m16);
   if (lane == 0) scale[row] = s;
   const bool finite = m16 < inf16<DT>(), nan_row = m16 > inf16<DT>();
   if constexpr (HELD) {
 #pragma unroll
     for (int u = 0; u < kRowRecipeHeld; ++u) {
       const uint32_t c = lane + 64 * u;
-      if (c < chunks) dst[c] = row_codes8<DT>(raw[u], s, finite, nan_row);
+      if (c < chunks) dst[c] = divided_codes8<DT>(raw[u], s, finite, nan_row);
     }
   } else {
-    for (uint32_t c = lane; c < chunks; c += 64) dst[c] = row_codes8<DT>(src[c], s, finite, nan_row);
+    for (uint32_t c = lane; c < chunks; c += 64) dst[c] = divided_codes8<DT>(src[c], s, finite, nan_row);
   }
 }
 
@@ -518,20 +520,12 @@ __global__ __launch_bounds__(256) void quant_fp8_rows_generic(const uint16_t* __
     m16 = a > m16 ? a : m16;
   }
   m16 = wave_max(m16);
-  const float s = row_scale_of<DT>(m16);
+  const float s = scale_of_amax16<DT>(m16);
   if (lane == 0) scale[row] = s;
   const bool finite = m16 < inf16<DT>(), nan_row = m16 > inf16<DT>();
   uint8_t* dst = q + (int64_t)row * cols;
   for (int64_t c = lane; c < cols; c += 64) {
-    const uint32_t h = src[c * sc];
-    uint32_t code;
-    if (finite) {
-      const float d = __builtin_amdgcn_fmed3f(__fdiv_rn(widen<DT>(h), s), -448.0f, 448.0f);
-      code = cvt4_f32(d, 0.f, 0.f, 0.f, 1.0f) & 0xFFu;
-    } else {
-      code = nonfinite_row_code<DT>(h, nan_row);
-    }
-    dst[c] = (uint8_t)code;
+    dst[c] = (uint8_t)divided_code1<DT>(src[c * sc], s, finite, nan_row);
   }
 }
 
@@ -618,7 +612,7 @@ extern "C" int km_quant_tensor(const void* x, int64_t rows, int64_t cols, int64_
   if (n > 0 && (!x || !q)) return km_fail(KM_ERR_ARG, "km_quant_tensor: null pointer");
   hipLaunchKernelGGL(fill_u32, dim3(1), dim3(1), 0, st, amax_workspace, 0u);
   int64_t want = (n / 8 + 255) / 256;
-  unsigned blocks = (unsigned)(want < 1 ? 1 : (want > 8192 ? 8192 : want));
+  unsigned blocks = (unsigned)(want < 1 ? 1 : (want > kTensorBlocks ? kTensorBlocks : want));
   const uint16_t* xp = (const uint16_t*)x;
   KM_DISPATCH_DT(dtype, {
     if (n > 0) hipLaunchKernelGGL(tensor_amax<DT>, dim3(blocks), dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, amax_workspace);
