@@ -3,7 +3,7 @@
 //   quant_mx_rows     MXFP8 along a unit-stride contraction axis (reference
 //                     src/kohakumoss_kernels/fp8/formats.py:94-99; the Triton kernel it
 //                     replaces is backends/triton/fp8/quantize.py:94-118)
-//   quant_mx_cols     MXFP8 of the transposed view (blocks run along the strided axis of
+//   quant_cols<MX>    MXFP8 of the transposed view (blocks run along the strided axis of
 //                     the input), what `quantize(x.t(), "mx")` computes for the input-
 //                     gradient weight copy (reference src/kohakumoss/quant/compute.py:63-66)
 //   quant_mx_generic  any strides, one thread per block of 32
@@ -115,6 +115,71 @@ __device__ __forceinline__ uint32_t amax16x8(const uint4& raw) {
   return m.x > m.y ? m.x : m.y;
 }
 
+// ---- fp32-scale recipes (per row, per tensor) ---------------------------------------------------
+// s = max(amax, 1e-12) / 448 and q = e4m3(clamp(x / s)), both IEEE fp32 divisions (reference
+// formats.py:41-45).
+__device__ __forceinline__ uint32_t wave_max(uint32_t m) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const uint32_t o = (uint32_t)__shfl_xor((int)m, off);
+    m = o > m ? o : m;
+  }
+  return m;
+}
+
+// Codes of a row (tensor) whose amax is infinite or NaN, where clamp-and-convert instructions and the
+// reference's host arithmetic part ways. Scale inf: finite x / inf is a signed zero, inf / inf
+// is NaN. Scale NaN: every quotient is NaN; the reference's host division hands back the
+// scale's NaN (code 0x7F) unless x is a NaN itself (code 0xFF, as for inf / inf).
+template <int DT>
+__device__ __forceinline__ uint32_t nonfinite_code(uint32_t h, bool nan_row) {
+  const uint32_t a = h & 0x7FFFu;
+  if (nan_row) return a > inf16<DT>() ? 0xFFu : 0x7Fu;
+  return a == inf16<DT>() ? 0xFFu : (h >> 8) & 0x80u;
+}
+
+template <int DT>
+__device__ __forceinline__ uint2 divided_codes8(const uint4& raw, float s, bool finite, bool nan_row) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  uint32_t out[2];
+  if (finite) {
+    float f[8];
+    widen8<DT>(raw, f);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = __builtin_amdgcn_fmed3f(__fdiv_rn(f[i], s), -448.0f, 448.0f);
+    out[0] = cvt4_f32(f[0], f[1], f[2], f[3], 1.0f);
+    out[1] = cvt4_f32(f[4], f[5], f[6], f[7], 1.0f);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      out[i] = nonfinite_code<DT>(w[2 * i] & 0xFFFFu, nan_row) | (nonfinite_code<DT>(w[2 * i] >> 16, nan_row) << 8) |
+               (nonfinite_code<DT>(w[2 * i + 1] & 0xFFFFu, nan_row) << 16) | (nonfinite_code<DT>(w[2 * i + 1] >> 16, nan_row) << 24);
+    }
+  }
+  return make_uint2(out[0], out[1]);
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t divided_code1(uint32_t h, float s, bool finite, bool nan_row) {
+  if (!finite) return nonfinite_code<DT>(h, nan_row);
+  const float d = __builtin_amdgcn_fmed3f(__fdiv_rn(widen<DT>(h), s), -448.0f, 448.0f);
+  return cvt4_f32(d, 0.f, 0.f, 0.f, 1.0f) & 0xFFu;
+}
+
+// scale from the largest 16-bit absolute-value pattern of a row
+template <int DT>
+__device__ __forceinline__ float scale_of_amax16(uint32_t m16) {
+  if (m16 > inf16<DT>()) return bits_f32(0x7FC00000u);
+  const uint32_t ab = widen_bits<DT>(m16);
+  return __fdiv_rn(bits_f32(ab > kAmaxFloorBits ? ab : kAmaxFloorBits), 448.0f);
+}
+
+// the same from the fp32 bits of an amax
+__device__ __forceinline__ float scale_of_amax_bits(uint32_t ab) {
+  if (ab > kInfBits) return bits_f32(0x7FC00000u);
+  return __fdiv_rn(bits_f32(ab > kAmaxFloorBits ? ab : kAmaxFloorBits), 448.0f);
+}
+
 // ---- rows: lane = 8 consecutive elements, quad = one block of 32 --------------------------
 // Group g (8 elements) of row g / groups_per_row; outputs are flat because q and the
 // scales are contiguous row-major. UNROLL independent 128-bit loads are in flight per lane.
@@ -199,10 +264,14 @@ constexpr int kColsTC = 128;  // columns of x per tile: 256-byte row segments
 constexpr int kColsPitch = kColsTC / 2 + 4;  // dwords per staged row (16-byte aligned rows)
 constexpr int kColsSkew = 8;  // extra dwords after each 32 rows: spreads the 8 blocks over banks
 
-template <int DT>
-__global__ __launch_bounds__(kColsThreads) void quant_mx_cols(
+// MX: one E8M0 scale per block of 32 rows, found here. !MX: one fp32 scale per column of x (per
+// row of q_t) from `col_amax`, the fp32 bits of each column's amax taken by an earlier pass;
+// rows may then be any multiple of 16.
+template <int DT, bool MX>
+__global__ __launch_bounds__(kColsThreads) void quant_cols(
     const uint16_t* __restrict__ x, int64_t ld, int64_t rows, int64_t cols,
-    uint8_t* __restrict__ q_t, uint8_t* __restrict__ scales_t, uint8_t* __restrict__ scales_km) {
+    uint8_t* __restrict__ q_t, uint8_t* __restrict__ scales_t, uint8_t* __restrict__ scales_km,
+    const uint32_t* __restrict__ col_amax) {
   __shared__ __attribute__((aligned(16))) uint32_t tile[kColsTR * kColsPitch + (kColsTR / 32) * kColsSkew];
   const int64_t r0 = (int64_t)blockIdx.y * kColsTR;
   const int64_t c0 = (int64_t)blockIdx.x * kColsTC;
@@ -247,10 +316,31 @@ __global__ __launch_bounds__(kColsThreads) void quant_mx_cols(
     const v2us a = __builtin_bit_cast(v2us, w[i] & 0x7FFF7FFFu), m = __builtin_bit_cast(v2us, mm);
     mm = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, m));
   }
+  uint32_t o0[8], o1[8];
+  if constexpr (!MX) {
+    const uint32_t ab0 = col_amax[c], ab1 = c + 1 < cols ? col_amax[c + 1] : 0u;
+    const float s0 = scale_of_amax_bits(ab0), s1 = scale_of_amax_bits(ab1);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t lo01 = __builtin_amdgcn_perm(w[4 * j + 1], w[4 * j], 0x05040100u), hi01 = __builtin_amdgcn_perm(w[4 * j + 1], w[4 * j], 0x07060302u);
+      const uint32_t lo23 = __builtin_amdgcn_perm(w[4 * j + 3], w[4 * j + 2], 0x05040100u), hi23 = __builtin_amdgcn_perm(w[4 * j + 3], w[4 * j + 2], 0x07060302u);
+      o0[j] = divided_codes8<DT>(make_uint4(lo01, lo23, 0, 0), s0, ab0 < kInfBits, ab0 > kInfBits).x;
+      o1[j] = divided_codes8<DT>(make_uint4(hi01, hi23, 0, 0), s1, ab1 < kInfBits, ab1 > kInfBits).x;
+    }
+    // rows % 16 == 0: the last block of a column may hold 16 rows only
+    uint4* d0 = reinterpret_cast<uint4*>(q_t + c * rows + rb);
+    d0[0] = make_uint4(o0[0], o0[1], o0[2], o0[3]);
+    if (rb + 32 <= rows) d0[1] = make_uint4(o0[4], o0[5], o0[6], o0[7]);
+    if (c + 1 < cols) {
+      uint4* d1 = reinterpret_cast<uint4*>(q_t + (c + 1) * rows + rb);
+      d1[0] = make_uint4(o1[0], o1[1], o1[2], o1[3]);
+      if (rb + 32 <= rows) d1[1] = make_uint4(o1[4], o1[5], o1[6], o1[7]);
+    }
+    return;
+  }
   const uint32_t m0 = mm & 0xFFFFu, m1 = mm >> 16;
   const uint32_t b0 = mx_biased_exponent(widen_bits<DT>(m0)), b1 = mx_biased_exponent(widen_bits<DT>(m1));
   const float s0 = bits_f32(b0 << 23), s1 = bits_f32(b1 << 23);
-  uint32_t o0[8], o1[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     // rows 4j .. 4j+3 of each column: regroup the halves so that a conversion sees one column
@@ -276,6 +366,54 @@ __global__ __launch_bounds__(kColsThreads) void quant_mx_cols(
     if (scales_t) scales_t[(c + 1) * nblk + lb] = (uint8_t)b1;
     if (scales_km) scales_km[scale_pack_offset(c + 1, lb, (cols + 127) >> 7)] = (uint8_t)b1;
   }
+}
+
+// fp32 bits of the abs-max of every column of a row-major [rows][cols] matrix, merged into
+// `col_amax` (zeroed beforehand) with one atomic max per column and workgroup. Tiles as above.
+__global__ void fill_u32_n(uint32_t* p, int64_t n, uint32_t v) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+template <int DT>
+__global__ __launch_bounds__(kColsThreads) void cols_amax(const uint16_t* __restrict__ x, int64_t ld, int64_t rows,
+                                                          int64_t cols, uint32_t* __restrict__ col_amax) {
+  constexpr int kLanesPerRow = kColsTC / 8, kRowGroups = kColsThreads / kLanesPerRow;
+  __shared__ uint32_t part[kRowGroups][kColsTC / 2 + 1];
+  const int64_t r0 = (int64_t)blockIdx.y * kColsTR;
+  const int64_t c0 = (int64_t)blockIdx.x * kColsTC;
+  const int cg = threadIdx.x % kLanesPerRow, rr = threadIdx.x / kLanesPerRow;
+  const int64_t c = c0 + cg * 8;
+  uint4 raw[kColsTR / kRowGroups];
+#pragma unroll
+  for (int i = 0; i < kColsTR / kRowGroups; ++i) {
+    const int64_t r = r0 + rr + kRowGroups * i;
+    raw[i] = make_uint4(0, 0, 0, 0);
+    if (r < rows && c < cols) raw[i] = *reinterpret_cast<const uint4*>(x + r * ld + c);
+  }
+  v2us m[4] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}};
+#pragma unroll
+  for (int i = 0; i < kColsTR / kRowGroups; ++i) {
+    const uint32_t w[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) m[k] = __builtin_elementwise_max(m[k], __builtin_bit_cast(v2us, w[k] & 0x7FFF7FFFu));
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) part[rr][cg * 4 + k] = __builtin_bit_cast(uint32_t, m[k]);
+  __syncthreads();
+  if (threadIdx.x < kColsTC / 2) {
+    v2us a = {0, 0};
+#pragma unroll 8
+    for (int g = 0; g < kRowGroups; ++g) a = __builtin_elementwise_max(a, __builtin_bit_cast(v2us, part[g][threadIdx.x]));
+    const int64_t cc = c0 + threadIdx.x * 2;
+    if (cc < cols && a.x != 0) atomicMax(col_amax + cc, widen_bits<DT>(a.x));
+    if (cc + 1 < cols && a.y != 0) atomicMax(col_amax + cc + 1, widen_bits<DT>(a.y));
+  }
+}
+
+__global__ void amax_bits_to_scales(uint32_t* p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = f32_bits(scale_of_amax_bits(p[i]));
 }
 
 // ---- generic: any strides, one thread per block ----------------------------------------------
@@ -312,65 +450,6 @@ __global__ __launch_bounds__(256) void scales_pack(const uint8_t* __restrict__ i
   if (i >= rows * blocks) return;
   const int64_t r = i / blocks, b = i - r * blocks;
   out[scale_pack_offset(r, b, (rows + 127) >> 7)] = in[i];
-}
-
-// ---- fp32-scale recipes (per row, per tensor) ---------------------------------------------------
-// s = max(amax, 1e-12) / 448 and q = e4m3(clamp(x / s)), both IEEE fp32 divisions (reference
-// formats.py:41-45).
-__device__ __forceinline__ uint32_t wave_max(uint32_t m) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    const uint32_t o = (uint32_t)__shfl_xor((int)m, off);
-    m = o > m ? o : m;
-  }
-  return m;
-}
-
-// Codes of a row (tensor) whose amax is infinite or NaN, where clamp-and-convert instructions and the
-// reference's host arithmetic part ways. Scale inf: finite x / inf is a signed zero, inf / inf
-// is NaN. Scale NaN: every quotient is NaN; the reference's host division hands back the
-// scale's NaN (code 0x7F) unless x is a NaN itself (code 0xFF, as for inf / inf).
-template <int DT>
-__device__ __forceinline__ uint32_t nonfinite_code(uint32_t h, bool nan_row) {
-  const uint32_t a = h & 0x7FFFu;
-  if (nan_row) return a > inf16<DT>() ? 0xFFu : 0x7Fu;
-  return a == inf16<DT>() ? 0xFFu : (h >> 8) & 0x80u;
-}
-
-template <int DT>
-__device__ __forceinline__ uint2 divided_codes8(const uint4& raw, float s, bool finite, bool nan_row) {
-  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-  uint32_t out[2];
-  if (finite) {
-    float f[8];
-    widen8<DT>(raw, f);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = __builtin_amdgcn_fmed3f(__fdiv_rn(f[i], s), -448.0f, 448.0f);
-    out[0] = cvt4_f32(f[0], f[1], f[2], f[3], 1.0f);
-    out[1] = cvt4_f32(f[4], f[5], f[6], f[7], 1.0f);
-  } else {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      out[i] = nonfinite_code<DT>(w[2 * i] & 0xFFFFu, nan_row) | (nonfinite_code<DT>(w[2 * i] >> 16, nan_row) << 8) |
-               (nonfinite_code<DT>(w[2 * i + 1] & 0xFFFFu, nan_row) << 16) | (nonfinite_code<DT>(w[2 * i + 1] >> 16, nan_row) << 24);
-    }
-  }
-  return make_uint2(out[0], out[1]);
-}
-
-template <int DT>
-__device__ __forceinline__ uint32_t divided_code1(uint32_t h, float s, bool finite, bool nan_row) {
-  if (!finite) return nonfinite_code<DT>(h, nan_row);
-  const float d = __builtin_amdgcn_fmed3f(__fdiv_rn(widen<DT>(h), s), -448.0f, 448.0f);
-  return cvt4_f32(d, 0.f, 0.f, 0.f, 1.0f) & 0xFFu;
-}
-
-// scale from the largest 16-bit absolute-value pattern of a row
-template <int DT>
-__device__ __forceinline__ float scale_of_amax16(uint32_t m16) {
-  if (m16 > inf16<DT>()) return bits_f32(0x7FC00000u);
-  const uint32_t ab = widen_bits<DT>(m16);
-  return __fdiv_rn(bits_f32(ab > kAmaxFloorBits ? ab : kAmaxFloorBits), 448.0f);
 }
 
 // ---- per-tensor recipe -----------------------------------------------------------------------
@@ -576,8 +655,8 @@ extern "C" int km_quant_mx(const void* x, int64_t rows, int64_t cols, int64_t st
     const int64_t mem_rows = cols, mem_cols = rows;
     dim3 grid((unsigned)((mem_cols + kColsTC - 1) / kColsTC), (unsigned)((mem_rows + kColsTR - 1) / kColsTR));
     if (grid.y > 65535u) return km_fail(KM_ERR_ARG, "km_quant_mx: tensor too large for the transposing kernel");
-    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL(quant_mx_cols<DT>, grid, dim3(kColsThreads), 0, st, xp, stride_col,
-                                             mem_rows, mem_cols, qp, sp, kp));
+    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL((quant_cols<DT, true>), grid, dim3(kColsThreads), 0, st, xp, stride_col,
+                                             mem_rows, mem_cols, qp, sp, kp, (const uint32_t*)nullptr));
   } else {
     const int64_t nb = rows * (cols / 32);
     KM_DISPATCH_DT(dtype, hipLaunchKernelGGL(quant_mx_generic<DT>, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, st,
@@ -640,6 +719,21 @@ extern "C" int km_quant_rows(const void* x, int64_t rows, int64_t cols, int64_t 
       else
         hipLaunchKernelGGL((quant_fp8_rows<DT, false>), grid, dim3(256), 0, st, xp, stride_row, chunks, (uint32_t)rows, (uint8_t*)q, scale_out);
     });
+  } else if (stride_row == 1 && aligned && (reinterpret_cast<uintptr_t>(q) & 15) == 0 && stride_col % 8 == 0 && stride_col >= rows &&
+             rows % 8 == 0 && cols % 16 == 0 && (cols + kColsTR - 1) / kColsTR <= 65535) {
+    // the memory is a row-major [cols][rows] matrix and q its transpose: column abs-max into
+    // scale_out (as fp32 bits), transposing conversion, then the bits become the scales
+    const int64_t mem_rows = cols, mem_cols = rows;
+    uint32_t* bits = reinterpret_cast<uint32_t*>(scale_out);
+    const dim3 tiles((unsigned)((mem_cols + kColsTC - 1) / kColsTC), (unsigned)((mem_rows + kColsTR - 1) / kColsTR));
+    const dim3 flat((unsigned)((rows + 255) / 256));
+    hipLaunchKernelGGL(fill_u32_n, flat, dim3(256), 0, st, bits, rows, 0u);
+    KM_DISPATCH_DT(dtype, {
+      hipLaunchKernelGGL(cols_amax<DT>, tiles, dim3(kColsThreads), 0, st, xp, stride_col, mem_rows, mem_cols, bits);
+      hipLaunchKernelGGL((quant_cols<DT, false>), tiles, dim3(kColsThreads), 0, st, xp, stride_col, mem_rows, mem_cols,
+                         (uint8_t*)q, (uint8_t*)nullptr, (uint8_t*)nullptr, (const uint32_t*)bits);
+    });
+    hipLaunchKernelGGL(amax_bits_to_scales, flat, dim3(256), 0, st, bits, rows);
   } else {
     KM_DISPATCH_DT(dtype, hipLaunchKernelGGL(quant_fp8_rows_generic<DT>, grid, dim3(256), 0, st, xp, stride_row, stride_col,
                                              (uint32_t)rows, cols, (uint8_t*)q, scale_out));

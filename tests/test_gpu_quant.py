@@ -178,7 +178,7 @@ def check_rows(x_cpu: torch.Tensor, view=lambda t: t):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("m,k", [(300, 1024), (5, 7), (1, 1), (64, 200), (33, 4096), (9, 4104), (130, 8192), (3, 12288)])
+@pytest.mark.parametrize("m,k", [(300, 1024), (5, 7), (1, 1), (64, 200), (33, 4096), (9, 4104), (130, 8192), (3, 12288), (256, 384), (48, 200), (1040, 136)])
 def test_row_recipe_bytes_equal_oracle(dtype, m, k):
     """Reference `tests/kernels/quant/test_fp8.py:61-82` for the row recipe: rows kept in
     registers (K <= 4096), rows read twice (K > 4096), ragged K (element-wise kernel) and the
@@ -228,11 +228,16 @@ def test_row_recipe_zero_tiny_inf_and_nan_rows():
     assert torch.equal(s.cpu()[keep].view(torch.int32), rs[keep].view(torch.int32))
     assert torch.equal(u8(q).cpu(), u8(rq))
     assert s.cpu()[0].item() == rs[0].item() == torch.tensor(1e-12).div(torch.tensor(448.0)).item()
+    # the same rows as columns of a [256, 8] matrix: the transposing kernels
+    xt = x.t().contiguous()
+    q2, s2 = native.quant_rows(xt.cuda().t())
+    assert torch.equal(u8(q2), u8(q)) and torch.equal(s2.view(torch.int32), s.view(torch.int32))
 
 
 def test_row_recipe_full_size_activation():
     x = outlier_operand()
     check_rows(x)
+    check_rows(x, view=lambda t: t.t())
 
 
 def test_row_recipe_argument_errors():
