@@ -138,15 +138,29 @@ __device__ __forceinline__ uint32_t nonfinite_code(uint32_t h, bool nan_row) {
   return a == inf16<DT>() ? 0xFFu : (h >> 8) & 0x80u;
 }
 
+// x / s as the IEEE division rounds it, from r = RN(1 / s): a product and two fused
+// corrections (each takes the exact remainder x - s q and adds remainder * r), the sign of x put
+// back for zeros. With r correctly rounded the second correction rounds correctly whenever the
+// first leaves q within one unit of the quotient; results differ from the division only far
+// below 2^-11, where every code is a signed zero. The GPU tests compare the kernels built on it
+// with the dividing element-wise kernels on every (amax, x) pair of 16-bit patterns.
+__device__ __forceinline__ float quotient(float x, float s, float r) {
+  float q = x * r;
+  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r, q);
+  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r, q);
+  return __builtin_copysignf(q, x);
+}
+
+// codes of the eight values of one 128-bit load; r = RN(1 / s)
 template <int DT>
-__device__ __forceinline__ uint2 divided_codes8(const uint4& raw, float s, bool finite, bool nan_row) {
+__device__ __forceinline__ uint2 divided_codes8(const uint4& raw, float s, float r, bool finite, bool nan_row) {
   const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
   uint32_t out[2];
   if (finite) {
     float f[8];
     widen8<DT>(raw, f);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = __builtin_amdgcn_fmed3f(__fdiv_rn(f[i], s), -448.0f, 448.0f);
+    for (int i = 0; i < 8; ++i) f[i] = __builtin_amdgcn_fmed3f(quotient(f[i], s, r), -448.0f, 448.0f);
     out[0] = cvt4_f32(f[0], f[1], f[2], f[3], 1.0f);
     out[1] = cvt4_f32(f[4], f[5], f[6], f[7], 1.0f);
   } else {
@@ -320,12 +334,13 @@ __global__ __launch_bounds__(kColsThreads) void quant_cols(
   if constexpr (!MX) {
     const uint32_t ab0 = col_amax[c], ab1 = c + 1 < cols ? col_amax[c + 1] : 0u;
     const float s0 = scale_of_amax_bits(ab0), s1 = scale_of_amax_bits(ab1);
+    const float r0 = __fdiv_rn(1.0f, s0), r1 = __fdiv_rn(1.0f, s1);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const uint32_t lo01 = __builtin_amdgcn_perm(w[4 * j + 1], w[4 * j], 0x05040100u), hi01 = __builtin_amdgcn_perm(w[4 * j + 1], w[4 * j], 0x07060302u);
       const uint32_t lo23 = __builtin_amdgcn_perm(w[4 * j + 3], w[4 * j + 2], 0x05040100u), hi23 = __builtin_amdgcn_perm(w[4 * j + 3], w[4 * j + 2], 0x07060302u);
-      o0[j] = divided_codes8<DT>(make_uint4(lo01, lo23, 0, 0), s0, ab0 < kInfBits, ab0 > kInfBits).x;
-      o1[j] = divided_codes8<DT>(make_uint4(hi01, hi23, 0, 0), s1, ab1 < kInfBits, ab1 > kInfBits).x;
+      o0[j] = divided_codes8<DT>(make_uint4(lo01, lo23, 0, 0), s0, r0, ab0 < kInfBits, ab0 > kInfBits).x;
+      o1[j] = divided_codes8<DT>(make_uint4(hi01, hi23, 0, 0), s1, r1, ab1 < kInfBits, ab1 > kInfBits).x;
     }
     // rows % 16 == 0: the last block of a column may hold 16 rows only
     uint4* d0 = reinterpret_cast<uint4*>(q_t + c * rows + rb);
@@ -509,6 +524,7 @@ __global__ __launch_bounds__(256) void tensor_cast(const uint16_t* __restrict__ 
   const uint32_t ab = *amax_bits;
   const bool finite = ab < kInfBits, nan_all = ab > kInfBits;
   const float s = nan_all ? bits_f32(0x7FC00000u) : __fdiv_rn(bits_f32(ab > kAmaxFloorBits ? ab : kAmaxFloorBits), 448.0f);
+  const float rcp = __fdiv_rn(1.0f, s);
   if (blockIdx.x == 0 && threadIdx.x == 0 && scale_out) *scale_out = s;
   const int64_t n = rows * cols;
   const bool dense = sc == 1 && sr == cols;
@@ -520,12 +536,12 @@ __global__ __launch_bounds__(256) void tensor_cast(const uint16_t* __restrict__ 
     int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
     for (; g + 3 * stride < nch; g += 4 * stride) {
       const uint4 r0 = src[g], r1 = src[g + stride], r2 = src[g + 2 * stride], r3 = src[g + 3 * stride];
-      dst[g] = divided_codes8<DT>(r0, s, finite, nan_all);
-      dst[g + stride] = divided_codes8<DT>(r1, s, finite, nan_all);
-      dst[g + 2 * stride] = divided_codes8<DT>(r2, s, finite, nan_all);
-      dst[g + 3 * stride] = divided_codes8<DT>(r3, s, finite, nan_all);
+      dst[g] = divided_codes8<DT>(r0, s, rcp, finite, nan_all);
+      dst[g + stride] = divided_codes8<DT>(r1, s, rcp, finite, nan_all);
+      dst[g + 2 * stride] = divided_codes8<DT>(r2, s, rcp, finite, nan_all);
+      dst[g + 3 * stride] = divided_codes8<DT>(r3, s, rcp, finite, nan_all);
     }
-    for (; g < nch; g += stride) dst[g] = divided_codes8<DT>(src[g], s, finite, nan_all);
+    for (; g < nch; g += stride) dst[g] = divided_codes8<DT>(src[g], s, rcp, finite, nan_all);
   } else {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
       const int64_t r = i / cols, c = i - r * cols;
@@ -570,16 +586,17 @@ __global__ __launch_bounds__(256) void quant_fp8_rows(const uint16_t* __restrict
   }
   m16 = wave_max(m16);
   const float s = scale_of_amax16<DT>(m16);
+  const float rcp = __fdiv_rn(1.0f, s);
   if (lane == 0) scale[row] = s;
   const bool finite = m16 < inf16<DT>(), nan_row = m16 > inf16<DT>();
   if constexpr (HELD) {
 #pragma unroll
     for (int u = 0; u < kRowRecipeHeld; ++u) {
       const uint32_t c = lane + 64 * u;
-      if (c < chunks) dst[c] = divided_codes8<DT>(raw[u], s, finite, nan_row);
+      if (c < chunks) dst[c] = divided_codes8<DT>(raw[u], s, rcp, finite, nan_row);
     }
   } else {
-    for (uint32_t c = lane; c < chunks; c += 64) dst[c] = divided_codes8<DT>(src[c], s, finite, nan_row);
+    for (uint32_t c = lane; c < chunks; c += 64) dst[c] = divided_codes8<DT>(src[c], s, rcp, finite, nan_row);
   }
 }
 

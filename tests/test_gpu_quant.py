@@ -234,6 +234,42 @@ def test_row_recipe_zero_tiny_inf_and_nan_rows():
     assert torch.equal(u8(q2), u8(q)) and torch.equal(s2.view(torch.int32), s.view(torch.int32))
 
 
+def pattern_rows(amax_patterns: torch.Tensor, dtype) -> torch.Tensor:
+    """Row i holds every 16-bit pattern of `dtype` whose magnitude is at most amax_patterns[i]
+    (the others are zero), so its amax is exactly that pattern: [len, 65536]."""
+    pats = torch.arange(0x10000, dtype=torch.int32, device=amax_patterns.device)
+    keep = (pats & 0x7FFF)[None, :] <= amax_patterns[:, None].to(torch.int32)
+    m = torch.where(keep, pats[None, :], torch.zeros((), dtype=torch.int32, device=pats.device))
+    return (m - (m >= 0x8000).to(torch.int32) * 0x10000).to(torch.int16).view(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_row_recipe_every_input_pattern_under_sampled_amax(dtype):
+    inf16 = 0x7F80 if dtype == torch.bfloat16 else 0x7C00
+    g = torch.Generator().manual_seed(5)
+    amax = torch.cat([torch.randint(1, inf16, (250,), generator=g), torch.tensor([0, 1, 0x80, inf16 - 1, inf16 // 2, inf16 // 2 + 1])])
+    check_rows(pattern_rows(amax, dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_row_recipe_vector_kernels_equal_the_dividing_kernel_on_every_pair(dtype):
+    """The vectorized kernels form x / s from a rounded reciprocal and two fused corrections;
+    the element-wise kernel (taken for a view that is not 16-byte aligned) divides. Every
+    (amax, x) pair of finite 16-bit patterns with |x| <= amax must give the same byte."""
+    inf16 = 0x7F80 if dtype == torch.bfloat16 else 0x7C00
+    chunk = 2048
+    for a0 in range(0, inf16, chunk):
+        amax = torch.arange(a0, min(a0 + chunk, inf16), device="cuda")
+        x = pattern_rows(amax, dtype)
+        wide = torch.zeros(x.shape[0], x.shape[1] + 8, dtype=dtype, device="cuda")
+        wide[:, 1:-7] = x
+        q_fast, s_fast = native.quant_rows(x)
+        q_div, s_div = native.quant_rows(wide[:, 1:-7])
+        assert torch.equal(s_fast.view(torch.int32), s_div.view(torch.int32))
+        assert torch.equal(u8(q_fast), u8(q_div)), f"amax patterns {a0}..{a0 + chunk}"
+        del x, wide, q_fast, q_div
+
+
 def test_row_recipe_full_size_activation():
     x = outlier_operand()
     check_rows(x)
