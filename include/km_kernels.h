@@ -97,6 +97,19 @@ int km_gemm_fp8_rows(const void *a, const float *sa, const void *b, const float 
                      const void *bias, void *c, int64_t M, int64_t N, int64_t K, int out_dtype,
                      int config, void *stream);
 
+/* int8 GEMM with int32 accumulation: C[m,n] = ((float(A B^T)[m,n] * sa[m]) * sb[n]) + bias[n], every
+ * product and the sum rounded to fp32 on its own and the result once to out_dtype, which makes
+ * the output equal, bit for bit, to the reference's eager int8 linear. A [M,K] and B [N,K] int8
+ * row-major, sa [M] fp32, sb [N] fp32 or NULL (ones; 16-byte aligned), bias [N] out_dtype or NULL.
+ * K % 256 == 0. Forward: A = Q(x), B = q, sb = weight scales; int8 input gradient: A = Q(dy * scale),
+ * B = q^T ([K,N] row-major copy), sb = NULL.
+ * Replaces torch._int_mm + the fp32 epilogue of int8.op.fwd_reference / dgrad_reference
+ * (src/kohakumoss_kernels/int8/op.py:40-60, int8/formats.py:39-52) and the Triton int8 GEMM
+ * (backends/triton/int8.py:47-133). */
+int km_gemm_i8_rows(const void *a, const float *sa, const void *b, const float *sb,
+                    const void *bias, void *c, int64_t M, int64_t N, int64_t K, int out_dtype,
+                    int config, void *stream);
+
 /* Weight-only forward: y[M,N] = (x[M,K] @ q[N,K]^T) * scale[N] + bias[N]; q int8 or e4m3fn
  * widened exactly to the activation dtype in registers, fp32 accumulation, scale and bias on
  * the accumulator, one rounding. Replaces Triton _fwd_kernel (backends/triton/quant.py:27-77). */

@@ -121,7 +121,10 @@ __device__ __forceinline__ uint32_t hidden_load_b32(const v4i& rsrc, int voffset
 // C[m0+wm+j*16+r16][n0+wn+t*16+4g .. +3]. Computes acc * post * row_scale[m] * col_scale[n] +
 // bias[n] in fp32 (either scale vector may be null), rounds once to the 16-bit output type. `bufs` are four LDS buffers of at least
 // `buf_bytes` each, free for staging (one per wavefront).
-template <int BM, int BN, int OUT, bool SCALED>
+// SCALED 0: acc + bias; 1: acc * (row * col scale) + bias, fused; 2: the accumulator holds int32
+// bits: ((float(acc) * row scale) * col scale) + bias with every product and the sum rounded
+// on its own, the order of the reference's int8 linear (src/kohakumoss_kernels/int8/op.py:45-48).
+template <int BM, int BN, int OUT, int SCALED>
 __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float post, const float* __restrict__ row_scale,
                                            const float* __restrict__ col_scale, const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N,
                                            int m0, int n0, uint8_t* buf0, uint8_t* buf1, uint8_t* buf2, uint8_t* buf3) {
@@ -132,7 +135,12 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
   const int r16 = lane & 15, g = lane >> 4;
   const bool has_bias = bias != nullptr;
   auto value = [&](float a, float rs, float cs, float b) __attribute__((always_inline)) {
-    if constexpr (SCALED) return a * (rs * cs) + b;
+    if constexpr (SCALED == 2) {
+#pragma clang fp contract(off)  // three roundings: a fused multiply-add would differ where the sum cancels
+      const float scaled_rows = (float)__builtin_bit_cast(int, a) * rs;
+      const float scaled = scaled_rows * cs;
+      return scaled + b;
+    } else if constexpr (SCALED == 1) return a * (rs * cs) + b;
     else return a + b;
   };
   if (m0 + BM <= M && n0 + BN <= N && (N & 7) == 0) {

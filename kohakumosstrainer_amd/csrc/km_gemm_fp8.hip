@@ -74,12 +74,26 @@ __device__ __forceinline__ void mfma_acc(v4f& c, const v8i& a, const v8i& b, int
 }
 #undef KM_MFMA_ASM
 
+// c += A(16x64) * B(64x16) of int8 codes with int32 accumulation (V_MFMA_I32_16X16X64_I8), the
+// accumulator tied in AGPRs as above (its registers hold int32 bits). Lane l supplies 16
+// consecutive K bytes of row l%16 in both operands, so each 16-byte half of a 128-byte-step
+// fragment (K bytes [16g, 16g+16) and [64+16g, 64+16g+16)) feeds one instruction: two of them
+// cover the step, in a K order that is the same for both operands.
+__device__ __forceinline__ void mfma_i8_acc(v4f& c, const v8i& a, const v8i& b) {
+  const v4i a_lo = __builtin_shufflevector(a, a, 0, 1, 2, 3), b_lo = __builtin_shufflevector(b, b, 0, 1, 2, 3);
+  const v4i a_hi = __builtin_shufflevector(a, a, 4, 5, 6, 7), b_hi = __builtin_shufflevector(b, b, 4, 5, 6, 7);
+  asm("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a_lo), "v"(b_lo));
+  asm("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a_hi), "v"(b_hi));
+}
+
 // A1: one A buffer instead of two (the A slab of step k+1 is requested at the top of step k,
 // once every wavefront holds the fragments of step k in registers, and waited for at its end).
 // Nothing stays in flight across the step boundary then, but the tile needs 3/4 of the LDS and,
 // with half the accumulators of the largest tile, two workgroups share a compute unit and fill
 // each other's waits, prologue and epilogue.
-template <int BM, int BN, bool MX, bool SCALE_KM, int OUT, bool A1>
+// I8: int8 codes on the int32 MFMA (no block scales), scale vectors applied in the reference's
+// order of roundings at the store.
+template <int BM, int BN, bool MX, bool SCALE_KM, int OUT, bool A1, bool I8>
 __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ As, const uint8_t* __restrict__ B,
     const uint8_t* __restrict__ Bs, const float* __restrict__ sa, const float* __restrict__ sb,
@@ -264,7 +278,9 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
       static_for<TM>([&](auto j_tag) __attribute__((always_inline)) {
         constexpr int j = decltype(j_tag)::value;
         constexpr int q = t * TM + j;  // position in the step's MFMA sequence
-        if constexpr (SCALE_KM)
+        if constexpr (I8)
+          mfma_i8_acc(acc[t][j], wcur, xf[j]);
+        else if constexpr (SCALE_KM)
           mfma_acc<t, j>(acc[t][j], wcur, xf[j], wscale[P][(t >> 2) % WS], xscale[P][(j >> 2) % XS]);
         else
           mfma_acc<0, 0>(acc[t][j], wcur, xf[j], wscale[P][t % WS], xscale[P][j % XS]);
@@ -306,7 +322,7 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
       }
       wcur = wnext;
     });
-    scale_commit(std::integral_constant<int, P ^ 1>{}, ks + 1 < nk ? 0xFFFFFFFFu : 0u);
+    if constexpr (!I8) scale_commit(std::integral_constant<int, P ^ 1>{}, ks + 1 < nk ? 0xFFFFFFFFu : 0u);
     __builtin_amdgcn_sched_barrier(0);
   };
   using set0_t = std::integral_constant<int, 0>;
@@ -319,12 +335,13 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
   if constexpr (!A1) dma_a(a_buf1, min(1, nk - 1));
   __builtin_amdgcn_s_waitcnt(kWaitVm0);
   __syncthreads();
-  scale_commit(set0_t{}, 0xFFFFFFFFu);
+  if constexpr (!I8) scale_commit(set0_t{}, 0xFFFFFFFFu);
 #pragma unroll
   for (int j = 0; j < TM; ++j) xf[j] = fragment(a_buf0, wm + j * 16 + r16);
   wcur = fragment(b_buf0, wn + r16);
 
-  // two steps per trip, one per buffer parity; an odd step count is padded with a zero-scaled step
+  // two steps per trip, one per buffer parity; an odd step count is padded with a zero-scaled
+  // step (int8 has no scale to zero: the host takes an even step count only)
   const int nsteps = (nk + 1) & ~1;
   for (int ks = 0; ks < nsteps; ks += 2) {
     step(a_buf0, A1 ? a_buf0 : a_buf1, b_buf0, b_buf1, ks, set0_t{});
@@ -349,11 +366,12 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
       post = sa[0] * sb[0];
     }
   }
+  constexpr int kEpilogue = I8 ? 2 : MX ? 0 : 1;
   if constexpr (A1) {
     static_assert(B_BYTES / 2 >= (BM < BN ? BM : BN) * 128, "epilogue staging in the halves of the B buffers");
-    store_tile<BM, BN, OUT, !MX>(acc, post, row_scale, col_scale, bias, C, M, N, m0, n0, b_buf0, b_buf0 + B_BYTES / 2, b_buf1, b_buf1 + B_BYTES / 2);
+    store_tile<BM, BN, OUT, kEpilogue>(acc, post, row_scale, col_scale, bias, C, M, N, m0, n0, b_buf0, b_buf0 + B_BYTES / 2, b_buf1, b_buf1 + B_BYTES / 2);
   } else {
-    store_tile<BM, BN, OUT, !MX>(acc, post, row_scale, col_scale, bias, C, M, N, m0, n0, a_buf0, a_buf1, b_buf0, b_buf1);
+    store_tile<BM, BN, OUT, kEpilogue>(acc, post, row_scale, col_scale, bias, C, M, N, m0, n0, a_buf0, a_buf1, b_buf0, b_buf1);
   }
 }
 
@@ -371,27 +389,27 @@ static const GemmConfig kGemmConfigs[] = {
 };
 constexpr int kNumGemmConfigs = sizeof(kGemmConfigs) / sizeof(kGemmConfigs[0]);
 
-template <int BM, int BN, bool MX, bool SCALE_KM, int OUT, bool A1 = false>
+template <int BM, int BN, bool MX, bool SCALE_KM, int OUT, bool A1, bool I8>
 static int launch_gemm(const void* a, const void* as, const void* b, const void* bs, const float* sa,
                        const float* sb, const void* bias, void* c, int M, int N, int K, int scale_vectors,
                        hipStream_t st) {
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  hipLaunchKernelGGL((gemm_fp8_kernel<BM, BN, MX, SCALE_KM, OUT, A1>), dim3(tiles), dim3(256), 0, st,
+  hipLaunchKernelGGL((gemm_fp8_kernel<BM, BN, MX, SCALE_KM, OUT, A1, I8>), dim3(tiles), dim3(256), 0, st,
                      (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b, (const uint8_t*)bs, sa, sb,
                      (const uint16_t*)bias, (uint16_t*)c, M, N, K, scale_vectors);
   return km_check_launch("km_gemm");
 }
 
-template <bool MX, bool SCALE_KM, int OUT>
+template <bool MX, bool SCALE_KM, int OUT, bool I8 = false>
 static int dispatch_config(int config, const void* a, const void* as, const void* b, const void* bs,
                            const float* sa, const float* sb, const void* bias, void* c, int M, int N,
                            int K, int scale_vectors, hipStream_t st) {
   switch (config) {
-    case 0: return launch_gemm<256, 256, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
-    case 1: return launch_gemm<128, 256, MX, SCALE_KM, OUT, true>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
-    case 2: return launch_gemm<256, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
-    case 3: return launch_gemm<128, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
-    case 4: return launch_gemm<64, 128, MX, SCALE_KM, OUT>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
+    case 0: return launch_gemm<256, 256, MX, SCALE_KM, OUT, false, I8>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
+    case 1: return launch_gemm<128, 256, MX, SCALE_KM, OUT, true, I8>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
+    case 2: return launch_gemm<256, 128, MX, SCALE_KM, OUT, false, I8>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
+    case 3: return launch_gemm<128, 128, MX, SCALE_KM, OUT, false, I8>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
+    case 4: return launch_gemm<64, 128, MX, SCALE_KM, OUT, false, I8>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
   }
   return km_fail(KM_ERR_ARG, "km_gemm: unknown config");
 }
@@ -484,4 +502,19 @@ extern "C" int km_gemm_fp8_rows(const void* a, const float* sa, const void* b, c
   if (out_dtype == KM_BF16)
     return dispatch_config<false, false, KM_BF16>(config, a, nullptr, b, nullptr, sa, sb, bias, c, (int)M, (int)N, (int)K, 1, st);
   return dispatch_config<false, false, KM_F16>(config, a, nullptr, b, nullptr, sa, sb, bias, c, (int)M, (int)N, (int)K, 1, st);
+}
+
+extern "C" int km_gemm_i8_rows(const void* a, const float* sa, const void* b, const float* sb,
+                               const void* bias, void* c, int64_t M, int64_t N, int64_t K,
+                               int out_dtype, int config, void* stream) {
+  int rc = check_gemm_args("km_gemm_i8_rows", a, b, c, M, N, K, out_dtype, config);
+  if (rc != KM_OK) return rc;
+  if (K % (2 * kStepBytes)) return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_i8_rows: K must be a multiple of 256");
+  if (M == 0 || N == 0) return KM_OK;
+  if (!sa) return km_fail(KM_ERR_ARG, "km_gemm_i8_rows: null row scale pointer");
+  if (reinterpret_cast<uintptr_t>(sb) & 15) return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_i8_rows: the column scales must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == KM_BF16)
+    return dispatch_config<false, false, KM_BF16, true>(config, a, nullptr, b, nullptr, sa, sb, bias, c, (int)M, (int)N, (int)K, 1, st);
+  return dispatch_config<false, false, KM_F16, true>(config, a, nullptr, b, nullptr, sa, sb, bias, c, (int)M, (int)N, (int)K, 1, st);
 }

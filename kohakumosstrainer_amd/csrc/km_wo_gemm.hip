@@ -223,9 +223,9 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   __builtin_amdgcn_sched_barrier(0);
 
   if constexpr (DGRAD)
-    store_tile<BM, BN, DT, false>(acc, 1.0f, nullptr, nullptr, nullptr, C, M, NO, m0, n0, a_buf0, a_buf1, b_buf0, b_buf1);
+    store_tile<BM, BN, DT, 0>(acc, 1.0f, nullptr, nullptr, nullptr, C, M, NO, m0, n0, a_buf0, a_buf1, b_buf0, b_buf1);
   else
-    store_tile<BM, BN, DT, true>(acc, 1.0f, nullptr, scale, bias, C, M, NO, m0, n0, a_buf0, a_buf1, b_buf0, b_buf1);
+    store_tile<BM, BN, DT, 1>(acc, 1.0f, nullptr, scale, bias, C, M, NO, m0, n0, a_buf0, a_buf1, b_buf0, b_buf1);
 }
 
 // Any shape, any alignment: one thread per output element (contraction lengths that are not a

@@ -34,6 +34,7 @@ EXPORTS = (
     "km_gemm_mx",
     "km_gemm_fp8_tensor",
     "km_gemm_fp8_rows",
+    "km_gemm_i8_rows",
     "km_wo_gemm_fwd",
     "km_wo_gemm_dgrad",
     "km_num_configs",
@@ -65,6 +66,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.km_gemm_mx.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_gemm_fp8_tensor.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_gemm_fp8_rows.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
+    lib.km_gemm_i8_rows.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_wo_gemm_fwd.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_wo_gemm_dgrad.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_num_configs.argtypes = [i32]
@@ -287,6 +289,29 @@ def gemm_fp8_rows(a: Tensor, sa: Tensor, b: Tensor, sb: Tensor, bias: Tensor | N
     sa, sb = sa.contiguous(), sb.contiguous()
     with torch.cuda.device(a.device):
         _check(load().km_gemm_fp8_rows(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), None if bias is None else bias.data_ptr(), c.data_ptr(), m, n, k, _dtype_code(out_dtype), config, _stream(a)))
+    return c
+
+
+def gemm_i8_rows(a: Tensor, sa: Tensor, b: Tensor, sb: Tensor | None, bias: Tensor | None, out_dtype: torch.dtype, config: int = 0) -> Tensor:
+    """`((int32(a b^T) * sa[:, None]) * sb[None, :]) + bias` rounded once to `out_dtype`; a `[M, K]`
+    and b `[N, K]` int8, sa `[M]` fp32, sb `[N]` fp32 or None (ones)."""
+    if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
+        raise ValueError(f"GEMM operands must be [M, K] and [N, K], got {tuple(a.shape)} and {tuple(b.shape)}")
+    if a.dtype != torch.int8 or b.dtype != torch.int8:
+        raise ValueError(f"int8 GEMM operands must be int8, got {a.dtype} and {b.dtype}")
+    m, k = a.shape
+    n = b.shape[0]
+    if tuple(sa.shape) != (m,) or sa.dtype != torch.float32 or (sb is not None and (tuple(sb.shape) != (n,) or sb.dtype != torch.float32)):
+        raise ValueError(f"int8 GEMM scales must be fp32 vectors [{m}] and [{n}]")
+    if bias is not None and (tuple(bias.shape) != (n,) or bias.dtype != out_dtype):
+        raise ValueError(f"bias must be [{n}] {out_dtype}, got {tuple(bias.shape)} {bias.dtype}")
+    dev = _on_gpu(a, b, sa, sb, bias)
+    a, b, sa = a.contiguous(), b.contiguous(), sa.contiguous()
+    sb = None if sb is None else sb.contiguous()
+    bias = None if bias is None else bias.contiguous()
+    c = torch.empty(m, n, device=dev, dtype=out_dtype)
+    with torch.cuda.device(dev):
+        _check(load().km_gemm_i8_rows(a.data_ptr(), sa.data_ptr(), b.data_ptr(), None if sb is None else sb.data_ptr(), None if bias is None else bias.data_ptr(), c.data_ptr(), m, n, k, _dtype_code(out_dtype), config, _stream(a)))
     return c
 
 
