@@ -71,6 +71,15 @@ int km_quant_tensor(const void *x, int64_t rows, int64_t cols, int64_t stride_ro
 int km_quant_rows(const void *x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,
                   int dtype, void *q, float *scale_out, void *stream);
 
+/* Per-row int8 quantizer of the int8 compute linear: v = x (* col_scale[c], in fp32, when col_scale
+ * is not NULL; [cols] fp32), scale_out[r] = max(amax of row r of v, 1e-12) / 127 (IEEE division),
+ * q[r, c] = clamp(round_half_even(v / scale_out[r]), +-127) (IEEE division). NaN inputs are outside
+ * the contract. Replaces int8.formats.quantize_rows(x, col_scale)
+ * (src/kohakumoss_kernels/int8/formats.py:21-38) and the Triton row quantizer
+ * (backends/triton/int8.py). */
+int km_quant_rows_i8(const void *x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,
+                     int dtype, const float *col_scale, void *q, float *scale_out, void *stream);
+
 /* C[M,N] = (A .* 2^(a_scale-127)) (B .* 2^(b_scale-127))^T + bias, A [M,K] and B [N,K] e4m3fn
  * row-major (K contiguous), scales E8M0 bytes, both in the layout scale_layout names
  * (KM_SCALES_ROWMAJOR: [M,K/32] / [N,K/32]; KM_SCALES_PACKED: see km_scales_pack), fp32 accumulation
@@ -101,7 +110,7 @@ int km_gemm_fp8_rows(const void *a, const float *sa, const void *b, const float 
  * product and the sum rounded to fp32 on its own and the result once to out_dtype, which makes
  * the output equal, bit for bit, to the reference's eager int8 linear. A [M,K] and B [N,K] int8
  * row-major, sa [M] fp32, sb [N] fp32 or NULL (ones; 16-byte aligned), bias [N] out_dtype or NULL.
- * K % 256 == 0. Forward: A = Q(x), B = q, sb = weight scales; int8 input gradient: A = Q(dy * scale),
+ * K % 128 == 0. Forward: A = Q(x), B = q, sb = weight scales; int8 input gradient: A = Q(dy * scale),
  * B = q^T ([K,N] row-major copy), sb = NULL.
  * Replaces torch._int_mm + the fp32 epilogue of int8.op.fwd_reference / dgrad_reference
  * (src/kohakumoss_kernels/int8/op.py:40-60, int8/formats.py:39-52) and the Triton int8 GEMM

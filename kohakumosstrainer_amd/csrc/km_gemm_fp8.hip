@@ -186,8 +186,10 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
   auto dma_a_pass = [&](uint8_t* buf, int koff, int i) __attribute__((always_inline)) {
     hidden_dma_b128(a_rsrc, lds_offset(buf) + i * 4096 + wave * 1024, ld_voff + i * pass_stride, koff);
   };
-  auto dma_b_pass = [&](uint8_t* buf, int koff, int i) __attribute__((always_inline)) {
-    hidden_dma_b128(b_rsrc, lds_offset(buf) + i * 4096 + wave * 1024, ld_voff + i * pass_stride, koff);
+  // `beyond` (0 or 2^31) pushes the per-lane offset past the descriptor's range: the pass then
+  // fills its LDS rows with zeros
+  auto dma_b_pass = [&](uint8_t* buf, int koff, int i, int beyond = 0) __attribute__((always_inline)) {
+    hidden_dma_b128(b_rsrc, lds_offset(buf) + i * 4096 + wave * 1024, ld_voff + i * pass_stride + beyond, koff);
   };
   auto dma_a = [&](uint8_t* buf, int ks) __attribute__((always_inline)) {
     const int koff = __builtin_amdgcn_readfirstlane(ks * kStepBytes);
@@ -261,6 +263,8 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
     const int next = min(ks + 1, nk - 1);
     const int koff_b = __builtin_amdgcn_readfirstlane(next * kStepBytes);
     const int koff_a = __builtin_amdgcn_readfirstlane(min(ks + (A1 ? 1 : 2), nk - 1) * kStepBytes);
+    // int8 has no scale to zero the padding step of an odd step count with: its B slab is zeros
+    const int b_beyond = I8 ? __builtin_amdgcn_readfirstlane(ks + 1 >= nk ? (int)0x80000000 : 0) : 0;
     scale_fetch(next);
     __builtin_amdgcn_sched_barrier(0);
     static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
@@ -291,7 +295,7 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
             constexpr int i = decltype(i_tag)::value;
             if constexpr (q == (A1 ? i : i * kBWindow / B_LD)) {
               __builtin_amdgcn_sched_barrier(0);
-              dma_b_pass(b_nxt, koff_b, i);
+              dma_b_pass(b_nxt, koff_b, i, b_beyond);
               __builtin_amdgcn_sched_barrier(0);
             }
           });
@@ -341,7 +345,7 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
   wcur = fragment(b_buf0, wn + r16);
 
   // two steps per trip, one per buffer parity; an odd step count is padded with a zero-scaled
-  // step (int8 has no scale to zero: the host takes an even step count only)
+  // step (int8: a step whose B slab is zeros)
   const int nsteps = (nk + 1) & ~1;
   for (int ks = 0; ks < nsteps; ks += 2) {
     step(a_buf0, A1 ? a_buf0 : a_buf1, b_buf0, b_buf1, ks, set0_t{});
@@ -509,7 +513,6 @@ extern "C" int km_gemm_i8_rows(const void* a, const float* sa, const void* b, co
                                int out_dtype, int config, void* stream) {
   int rc = check_gemm_args("km_gemm_i8_rows", a, b, c, M, N, K, out_dtype, config);
   if (rc != KM_OK) return rc;
-  if (K % (2 * kStepBytes)) return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_i8_rows: K must be a multiple of 256");
   if (M == 0 || N == 0) return KM_OK;
   if (!sa) return km_fail(KM_ERR_ARG, "km_gemm_i8_rows: null row scale pointer");
   if (reinterpret_cast<uintptr_t>(sb) & 15) return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_i8_rows: the column scales must be 16-byte aligned");

@@ -9,6 +9,8 @@
 //   quant_mx_generic  any strides, one thread per block of 32
 //   tensor_amax / tensor_cast   per-tensor recipe (reference formats.py:77-79,
 //                     Triton quantize.py:86-91,161-168)
+//   quant_i8_rows     int8 per-row quantizer of the int8 compute linear (reference
+//                     src/kohakumoss_kernels/int8/formats.py:21-38)
 //   quant_fp8_rows    per-row recipe, one fp32 scale per row (reference formats.py:80-82,
 //                     Triton quantize.py:64-84,151-158)
 //
@@ -625,6 +627,121 @@ __global__ __launch_bounds__(256) void quant_fp8_rows_generic(const uint16_t* __
   }
 }
 
+// ---- int8 per-row quantizer ----------------------------------------------------------------------
+// s[r] = max(amax_r, 1e-12) / 127 and q = clamp(round_half_even(x / s[r]), +-127), IEEE fp32
+// divisions, the columns multiplied by `col_scale` first (in fp32) when given (reference
+// src/kohakumoss_kernels/int8/formats.py:21-38; Triton backends/triton/int8.py). One wavefront
+// per row; NaN inputs are outside the contract (the reference's cast of NaN to int8 is
+// platform-defined).
+__device__ __forceinline__ uint32_t i8_code(float v, float s) {
+  const float r = __builtin_amdgcn_fmed3f(__builtin_rintf(__fdiv_rn(v, s)), -127.0f, 127.0f);
+  return (uint32_t)(int)r & 0xFFu;
+}
+
+template <int DT>
+__device__ __forceinline__ void scaled8(const uint4& raw, const float* __restrict__ col_scale, uint32_t chunk, float (&f)[8]) {
+  widen8<DT>(raw, f);
+  if (col_scale != nullptr) {
+    const float4 c0 = reinterpret_cast<const float4*>(col_scale)[2 * chunk], c1 = reinterpret_cast<const float4*>(col_scale)[2 * chunk + 1];
+    f[0] *= c0.x; f[1] *= c0.y; f[2] *= c0.z; f[3] *= c0.w;
+    f[4] *= c1.x; f[5] *= c1.y; f[6] *= c1.z; f[7] *= c1.w;
+  }
+}
+
+__device__ __forceinline__ uint32_t amax_bits_of8(const float (&f)[8]) {
+  uint32_t m = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const uint32_t a = f32_bits(f[i]) & kAbsMask;
+    m = a > m ? a : m;
+  }
+  return m;
+}
+
+__device__ __forceinline__ float i8_scale_of(uint32_t amax_bits) {
+  return __fdiv_rn(bits_f32(amax_bits > kAmaxFloorBits ? amax_bits : kAmaxFloorBits), 127.0f);
+}
+
+template <int DT, bool HELD>
+__global__ __launch_bounds__(256) void quant_i8_rows(const uint16_t* __restrict__ x, int64_t ld, uint32_t chunks, uint32_t rows,
+                                                     const float* __restrict__ col_scale, uint8_t* __restrict__ q,
+                                                     float* __restrict__ scale) {
+  const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const uint32_t lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const uint4* src = reinterpret_cast<const uint4*>(x + (uint64_t)row * (uint64_t)ld);
+  uint2* dst = reinterpret_cast<uint2*>(q + (uint64_t)row * chunks * 8);
+  uint4 raw[HELD ? kRowRecipeHeld : 1];
+  uint32_t m = 0;
+  float f[8];
+  if constexpr (HELD) {
+#pragma unroll
+    for (int u = 0; u < kRowRecipeHeld; ++u) {
+      const uint32_t c = lane + 64 * u;
+      raw[u] = c < chunks ? src[c] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < kRowRecipeHeld; ++u) {
+      const uint32_t c = lane + 64 * u;
+      if (c < chunks) {
+        scaled8<DT>(raw[u], col_scale, c, f);
+        const uint32_t a = amax_bits_of8(f);
+        m = a > m ? a : m;
+      }
+    }
+  } else {
+    for (uint32_t c = lane; c < chunks; c += 64) {
+      scaled8<DT>(src[c], col_scale, c, f);
+      const uint32_t a = amax_bits_of8(f);
+      m = a > m ? a : m;
+    }
+  }
+  m = wave_max(m);
+  const float s = i8_scale_of(m);
+  if (lane == 0) scale[row] = s;
+  auto codes = [&](const uint4& r, uint32_t c) __attribute__((always_inline)) {
+    scaled8<DT>(r, col_scale, c, f);
+    const uint32_t lo = i8_code(f[0], s) | (i8_code(f[1], s) << 8) | (i8_code(f[2], s) << 16) | (i8_code(f[3], s) << 24);
+    const uint32_t hi = i8_code(f[4], s) | (i8_code(f[5], s) << 8) | (i8_code(f[6], s) << 16) | (i8_code(f[7], s) << 24);
+    return make_uint2(lo, hi);
+  };
+  if constexpr (HELD) {
+#pragma unroll
+    for (int u = 0; u < kRowRecipeHeld; ++u) {
+      const uint32_t c = lane + 64 * u;
+      if (c < chunks) dst[c] = codes(raw[u], c);
+    }
+  } else {
+    for (uint32_t c = lane; c < chunks; c += 64) dst[c] = codes(src[c], c);
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void quant_i8_rows_generic(const uint16_t* __restrict__ x, int64_t sr, int64_t sc, uint32_t rows,
+                                                             int64_t cols, const float* __restrict__ col_scale,
+                                                             uint8_t* __restrict__ q, float* __restrict__ scale) {
+  const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const uint32_t lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const uint16_t* src = x + (int64_t)row * sr;
+  uint32_t m = 0;
+  for (int64_t c = lane; c < cols; c += 64) {
+    float v = widen<DT>(src[c * sc]);
+    if (col_scale != nullptr) v *= col_scale[c];
+    const uint32_t a = f32_bits(v) & kAbsMask;
+    m = a > m ? a : m;
+  }
+  m = wave_max(m);
+  const float s = i8_scale_of(m);
+  if (lane == 0) scale[row] = s;
+  uint8_t* dst = q + (int64_t)row * cols;
+  for (int64_t c = lane; c < cols; c += 64) {
+    float v = widen<DT>(src[c * sc]);
+    if (col_scale != nullptr) v *= col_scale[c];
+    dst[c] = (uint8_t)i8_code(v, s);
+  }
+}
+
 }  // namespace km
 
 using namespace km;
@@ -756,4 +873,31 @@ extern "C" int km_quant_rows(const void* x, int64_t rows, int64_t cols, int64_t 
                                              (uint32_t)rows, cols, (uint8_t*)q, scale_out));
   }
   return km_check_launch("km_quant_rows");
+}
+
+extern "C" int km_quant_rows_i8(const void* x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,
+                                int dtype, const float* col_scale, void* q, float* scale_out, void* stream) {
+  if (dtype != KM_BF16 && dtype != KM_F16) return km_fail(KM_ERR_ARG, "km_quant_rows_i8: dtype must be bf16 or f16");
+  if (rows < 0 || cols < 0) return km_fail(KM_ERR_ARG, "km_quant_rows_i8: negative shape");
+  if (rows == 0) return KM_OK;
+  if (rows > 0x7FFFFFFFll) return km_fail(KM_ERR_ARG, "km_quant_rows_i8: too many rows");
+  if (!scale_out || (cols > 0 && (!x || !q))) return km_fail(KM_ERR_ARG, "km_quant_rows_i8: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const uint16_t* xp = (const uint16_t*)x;
+  const dim3 grid((unsigned)((rows + 3) / 4));
+  const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0 &&
+                       (reinterpret_cast<uintptr_t>(col_scale) & 15) == 0;
+  if (stride_col == 1 && aligned && cols % 8 == 0 && stride_row % 8 == 0 && stride_row >= cols && cols / 8 <= 0x7FFFFFFFll) {
+    const uint32_t chunks = (uint32_t)(cols / 8);
+    KM_DISPATCH_DT(dtype, {
+      if (chunks <= 64u * kRowRecipeHeld)
+        hipLaunchKernelGGL((quant_i8_rows<DT, true>), grid, dim3(256), 0, st, xp, stride_row, chunks, (uint32_t)rows, col_scale, (uint8_t*)q, scale_out);
+      else
+        hipLaunchKernelGGL((quant_i8_rows<DT, false>), grid, dim3(256), 0, st, xp, stride_row, chunks, (uint32_t)rows, col_scale, (uint8_t*)q, scale_out);
+    });
+  } else {
+    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL(quant_i8_rows_generic<DT>, grid, dim3(256), 0, st, xp, stride_row, stride_col,
+                                             (uint32_t)rows, cols, col_scale, (uint8_t*)q, scale_out));
+  }
+  return km_check_launch("km_quant_rows_i8");
 }

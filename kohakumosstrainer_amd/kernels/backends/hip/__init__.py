@@ -9,4 +9,4 @@ _why = native.available()
 if _why is not None:
     raise RuntimeError(_why)
 
-from kohakumosstrainer_amd.kernels.backends.hip import fp8_linear, quant  # noqa: E402,F401
+from kohakumosstrainer_amd.kernels.backends.hip import fp8_linear, int8, quant  # noqa: E402,F401

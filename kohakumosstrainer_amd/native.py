@@ -31,6 +31,7 @@ EXPORTS = (
     "km_scales_pack",
     "km_quant_tensor",
     "km_quant_rows",
+    "km_quant_rows_i8",
     "km_gemm_mx",
     "km_gemm_fp8_tensor",
     "km_gemm_fp8_rows",
@@ -63,6 +64,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.km_scales_pack.argtypes = [p, i64, i64, p, p]
     lib.km_quant_tensor.argtypes = [p, i64, i64, i64, i64, i32, p, p, p, p]
     lib.km_quant_rows.argtypes = [p, i64, i64, i64, i64, i32, p, p, p]
+    lib.km_quant_rows_i8.argtypes = [p, i64, i64, i64, i64, i32, p, p, p, p]
     lib.km_gemm_mx.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_gemm_fp8_tensor.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_gemm_fp8_rows.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
@@ -220,6 +222,24 @@ def quant_rows(x: Tensor) -> tuple[Tensor, Tensor]:
     with torch.cuda.device(x.device):
         _check(load().km_quant_rows(x.data_ptr(), rows, k, x.stride(0), x.stride(1), _dtype_code(x.dtype), q.data_ptr(), s.data_ptr(), _stream(x)))
     return q.view(E4M3), s
+
+
+def quant_rows_i8(x: Tensor, col_scale: Tensor | None = None) -> tuple[Tensor, Tensor]:
+    """`(q int8 [rows, K], scale fp32 [rows])` of the int8 compute linear, the columns of x times
+    `col_scale` [K] (fp32) first when given."""
+    if x.dim() != 2:
+        raise ValueError(f"int8 operand must be 2-D, got {tuple(x.shape)}")
+    _on_gpu(x, col_scale)
+    rows, k = x.shape
+    if col_scale is not None:
+        if tuple(col_scale.shape) != (k,):
+            raise ValueError(f"col_scale must be [{k}], got {tuple(col_scale.shape)}")
+        col_scale = col_scale.to(torch.float32).contiguous()
+    q = torch.empty(rows, k, device=x.device, dtype=torch.int8)
+    s = torch.empty(rows, device=x.device, dtype=torch.float32)
+    with torch.cuda.device(x.device):
+        _check(load().km_quant_rows_i8(x.data_ptr(), rows, k, x.stride(0), x.stride(1), _dtype_code(x.dtype), None if col_scale is None else col_scale.data_ptr(), q.data_ptr(), s.data_ptr(), _stream(x)))
+    return q, s
 
 
 # ---- GEMMs --------------------------------------------------------------------------------

@@ -37,7 +37,7 @@ def n_configs():
 
 
 @pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
-@pytest.mark.parametrize("m,n,k", [(200, 384, 256), (1000, 512, 768), (1, 128, 256), (513, 200, 1024), (61, 136, 4096)])
+@pytest.mark.parametrize("m,n,k", [(200, 384, 256), (1000, 512, 768), (1, 128, 128), (513, 200, 1152), (61, 136, 4096), (300, 256, 384)])
 def test_i8_gemm_every_config_is_exact(dtype, m, n, k):
     a, b, sa, sb, g = problem(m, n, k, seed=m + n)
     bias = (torch.randn(n, generator=g) * 0.1).to(dtype)
@@ -53,7 +53,7 @@ def test_i8_gemm_every_config_is_exact(dtype, m, n, k):
 def test_i8_gemm_one_hot_operands_pin_the_k_order():
     """A single +-1 per row of `a` picks one column of b^T: any K permutation that differs
     between the two operands, or a dropped half of a 128-byte step, shows."""
-    k, n = 512, 128
+    k, n = 640, 128
     g = torch.Generator().manual_seed(9)
     b = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8)
     a = torch.zeros(k, k, dtype=torch.int8)
@@ -75,10 +75,10 @@ def test_i8_gemm_extreme_codes_do_not_overflow():
 
 
 def test_i8_gemm_argument_errors():
-    a = torch.zeros(64, 128, dtype=torch.int8, device="cuda")
+    a = torch.zeros(64, 192, dtype=torch.int8, device="cuda")
     s = torch.ones(64, device="cuda")
     with pytest.raises(native.KernelError):
-        native.gemm_i8_rows(a, s, a, s, None, torch.bfloat16, 0)  # K % 256
+        native.gemm_i8_rows(a, s, a, s, None, torch.bfloat16, 0)  # K % 128
     a = torch.zeros(64, 256, dtype=torch.int8, device="cuda")
     with pytest.raises(native.KernelError):
         native.gemm_i8_rows(a, s, a, s, None, torch.bfloat16, 99)

@@ -1,0 +1,132 @@
+"""int8 compute linear on the GPU through the C ABI and the registry: the HIP per-row quantizer
+against the CPU oracle byte for byte, the op's forward and int8 input gradient against the
+oracle bit for bit (the integer accumulation is exact and the epilogue rounds in the eager
+path's order), the 16-bit input gradient by the weight-only tolerance. Mirrors reference
+`tests/kernels/quant/test_int8_linear.py:163-260` (every backend against the eager reference and
+fp64, both dgrad modes, bf16 and fp16, under torch.compile)."""
+
+import pytest
+import torch
+
+from kohakumosstrainer_amd import native
+from kohakumosstrainer_amd.kernels import registry, tuning
+from oracle import int8 as oi
+from oracle import stats as oracle_stats
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+DTYPES = (torch.bfloat16, torch.float16)
+
+
+@pytest.fixture(autouse=True)
+def untimed():
+    tuning.set_mode("off")
+    tuning.reset()
+    yield
+    tuning.set_mode("table")
+    tuning.reset()
+
+
+def activations(m, k, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(m, k, generator=g) * torch.logspace(-3, 2, m)[:, None]
+    if m > 2:
+        x[1] = 0.0
+        x[2, : min(k, 5)] = torch.tensor([127.0, 0.5, 1.5, -2.5, -127.0])[: min(k, 5)]
+        x[2, min(k, 5):] = 0.0
+    return x.to(dtype), g
+
+
+def check_rows(x_cpu, col=None, view=lambda t: t):
+    q, s = native.quant_rows_i8(view(x_cpu.cuda()), None if col is None else col.cuda())
+    rq, rs = oi.quantize_rows(view(x_cpu), col)
+    assert q.dtype == torch.int8 and s.dtype == torch.float32 and q.shape == rq.shape and q.is_contiguous()
+    assert torch.equal(s.cpu().view(torch.int32), rs.view(torch.int32)), "scale bits"
+    assert torch.equal(q.cpu(), rq), "codes"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,k", [(300, 1024), (5, 7), (1, 1), (64, 200), (33, 4096), (9, 4104), (130, 8192)])
+def test_quantizer_bytes_equal_oracle(dtype, m, k):
+    x, g = activations(m, k, dtype, seed=m)
+    col = torch.rand(k, generator=g) * 1e-2 + 1e-5
+    check_rows(x)
+    check_rows(x, col)
+    check_rows(x, view=lambda t: t.t(), col=torch.rand(m, generator=g) + 0.1)
+    if k >= 16:
+        check_rows(x, view=lambda t: t[:, 8:], col=col[8:])
+        check_rows(x, view=lambda t: t[:, 1 : k - 1])
+
+
+def test_quantizer_half_even_known_answers_and_floor():
+    x = torch.tensor([[127.0, 0.5, 1.5, -2.5, -127.0, 0.0, 0.0, 0.0], [0.0] * 8]).to(torch.bfloat16)
+    q, s = native.quant_rows_i8(x.cuda())
+    assert q.cpu()[0].tolist() == [127, 0, 2, -2, -127, 0, 0, 0] and q.cpu()[1].tolist() == [0] * 8
+    assert s.cpu()[0].item() == 1.0 and s.cpu()[1].item() == oi.row_scale(torch.zeros(1)).item()
+
+
+def test_quantizer_every_bf16_pattern_under_sampled_amax():
+    g = torch.Generator().manual_seed(6)
+    amax = torch.cat([torch.randint(1, 0x7F80, (120,), generator=g), torch.tensor([0, 1, 0x80, 0x7F7F])])
+    pats = torch.arange(0x10000, dtype=torch.int32)
+    keep = (pats & 0x7FFF)[None, :] <= amax[:, None].to(torch.int32)
+    m = torch.where(keep, pats[None, :], torch.zeros((), dtype=torch.int32))
+    x = (m - (m >= 0x8000).to(torch.int32) * 0x10000).to(torch.int16).view(torch.bfloat16)
+    check_rows(x)
+
+
+def test_quantizer_full_size():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(16384, 3072, generator=g)
+    mask = torch.rand(16384, 3072, generator=g) < 1e-3
+    x[mask] = (torch.randn(16384, 3072, generator=g) * 50)[mask]
+    check_rows(x.to(torch.bfloat16))
+
+
+def weight(n, k, g):
+    w = torch.randn(n, k, generator=g) * 0.05
+    scale = (w.abs().amax(dim=1).clamp_min(1e-12) / 127.0).float()
+    return torch.round(w / scale[:, None]).clamp(-127, 127).to(torch.int8), scale
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(200, 256, 256), (513, 384, 1024), (5, 512, 768), (61, 2048, 4096)])
+def test_int8_linear_forward_and_grads(dtype, m, n, k):
+    g = torch.Generator().manual_seed(m)
+    q, scale = weight(n, k, g)
+    x = torch.randn(m, k, generator=g).to(dtype)
+    bias = (torch.randn(n, generator=g) * 0.1).to(dtype)
+    dy = torch.randn(m, n, generator=g).to(dtype)
+    for mode in oi.DGRAD:
+        op = registry.resolve("int8_linear", DEV, dtype, group=0, dgrad=mode)
+        assert op.backend == "hip"
+        xd = x.to(DEV).requires_grad_(True)
+        bd = bias.to(DEV).requires_grad_(True)
+        y = op(xd, q.to(DEV), scale.to(DEV), bd, 0, mode)
+        y.backward(dy.to(DEV))
+        assert torch.equal(y.detach().cpu(), oi.forward(x, q, scale, bias)), "forward bits"
+        want_dx = oi.dgrad(dy, q, scale, mode)
+        if mode == "int8":
+            assert torch.equal(xd.grad.cpu(), want_dx), "int8 input gradient bits"
+        else:
+            exact = dy.double() @ (q.double() * scale.double()[:, None])
+            oracle_stats.assert_no_regression(xd.grad.cpu(), want_dx, exact, name="16bit dgrad")
+        assert torch.equal(bd.grad.cpu(), dy.float().sum(0).to(dtype))
+    no_bias = registry.resolve("int8_linear", DEV, dtype, group=0, dgrad="int8")(x.to(DEV), q.to(DEV), scale.to(DEV), None, 0, "int8")
+    assert torch.equal(no_bias.cpu(), oi.forward(x, q, scale, None)) and not no_bias.requires_grad
+
+
+def test_int8_linear_leading_dims_compile_and_support():
+    g = torch.Generator().manual_seed(2)
+    q, scale = weight(256, 512, g)
+    x = torch.randn(4, 32, 512, generator=g).to(torch.bfloat16)
+    op = registry.resolve("int8_linear", DEV, torch.bfloat16, group=0, dgrad="int8")
+    y = op(x.to(DEV), q.to(DEV), scale.to(DEV), None, 0, "int8")
+    assert y.shape == (4, 32, 256)
+    assert torch.equal(y.cpu().reshape(128, 256), oi.forward(x.reshape(128, 512), q, scale, None))
+    compiled = torch.compile(lambda t: op(t, q.to(DEV), scale.to(DEV), None, 0, "int8"), fullgraph=True)
+    assert torch.equal(compiled(x.to(DEV)), y)
+    assert "not built" in registry.available("int8_linear", DEV, torch.bfloat16, group=256, dgrad="int8")["hip"]
+    assert "not in" in registry.available("int8_linear", DEV, torch.bfloat16, group=0, dgrad="fp4")["hip"]
+    with pytest.raises(ValueError):
+        op(x.to(DEV)[..., :320], q.to(DEV)[:, :320], scale.to(DEV), None, 0, "int8")  # K % 128
