@@ -81,9 +81,20 @@ def cpu_baseline(x, wq, ws, bias):
 
 def other_configs(dev, reps):
     """Device time of the other kernels of the path at their benchmark shapes (event-timed,
-    back to back): weight-only int8 / e4m3 GEMMs and the frozen-base MXFP8 forward + input
-    gradient of the adapter-training shape."""
+    back to back): weight-only int8 / e4m3 GEMMs, the frozen-base MXFP8 forward + input
+    gradient of the adapter-training shape, and the row-recipe fp8 and int8 compute linears at
+    the headline shape."""
+    import time
+
     from kohakumosstrainer_amd import native
+
+    timed_raw = event_ms
+
+    def event_ms(fn, reps):  # noqa: F811  (each measurement starts from sustained clocks)
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 0.05:
+            fn()
+        return timed_raw(fn, reps)
 
     g = torch.Generator(device="cpu").manual_seed(0)
     out = {}
@@ -155,6 +166,28 @@ def other_configs(dev, reps):
     out["row_recipe_M16384_K3072_N9216"] = {
         "quant_rows_us": qt * 1e3, "quant_rows_GBps": (m * k * 3 + m * 4) / qt / 1e6, "hbm_peak_GBps": HBM_PEAK_GBS,
         "gemm_ms": gt, "gemm_TFLOPs": flop / gt / 1e9, "step_ms": st, "step_TFLOPs": flop / st / 1e9, "peak_TFLOPs": FP8_PEAK_TFLOPS,
+    }
+    # int8 compute linear (per-row int8 activations, int8 MFMA GEMM, int32 accumulation), same shape
+    w_scale = (w.float().abs().amax(1).clamp_min(1e-12) / 127.0)
+    w8 = torch.round(w.float() / w_scale[:, None]).clamp_(-127, 127).to(torch.int8)
+    x8, x8s = native.quant_rows_i8(x)
+    q8buf = torch.empty(m, k, dtype=torch.int8, device=dev)
+
+    def quant8_only():
+        lib.km_quant_rows_i8(x.data_ptr(), m, k, k, 1, native.KM_BF16, None, q8buf.data_ptr(), sbuf.data_ptr(), stream)
+
+    def int8_step():
+        aq, sa = native.quant_rows_i8(x)
+        return native.gemm_i8_rows(aq, sa, w8, w_scale, bias, torch.bfloat16, 0)
+
+    quant8_only()
+    int8_step()
+    qt = event_ms(quant8_only, reps)
+    gt = event_ms(lambda: native.gemm_i8_rows(x8, x8s, w8, w_scale, bias, torch.bfloat16, 0), reps)
+    st = event_ms(int8_step, reps)
+    out["int8_compute_M16384_K3072_N9216"] = {
+        "quant_rows_us": qt * 1e3, "quant_rows_GBps": (m * k * 3 + m * 4) / qt / 1e6, "hbm_peak_GBps": HBM_PEAK_GBS,
+        "gemm_ms": gt, "gemm_TOPs": flop / gt / 1e9, "step_ms": st, "step_TOPs": flop / st / 1e9, "peak_TOPs": 5000.0,
     }
     return out
 

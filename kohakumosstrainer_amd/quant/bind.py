@@ -1,5 +1,5 @@
 """Binding quantized linears to their compute device and dtype after a placement (reference
-`src/kohakumoss/quant/bind.py:14-40`)."""
+`src/kohakumoss/quant/bind.py:14-40`; W4A8 and embedding bases are outside this path)."""
 
 import torch
 from torch import nn
@@ -16,6 +16,15 @@ def rebind_quant(module: nn.Module, device, dtype, autograd: bool = True) -> Non
             m.bind(dtype, device, autograd=autograd)
         elif isinstance(m, QuantWeight):
             m.bind(dtype, device)
+
+
+def set_int8_compute(module: nn.Module, dgrad: str) -> int:
+    """Select int8 compute (the `int8_linear` op with input-gradient mode `dgrad`) on every int8
+    base inside `module`; it takes effect at their next `bind`. Returns how many were switched."""
+    switched = [m for m in module.modules() if isinstance(m, QuantWeight) and m.fmt == "int8"]
+    for m in switched:
+        m.int8_dgrad = dgrad
+    return len(switched)
 
 
 def work_device(device) -> torch.device:

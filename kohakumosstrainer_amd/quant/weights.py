@@ -4,9 +4,10 @@ int8: q = round(w / s) clamped to [-127, 127], s = max|w_row| / 127.
 fp8 (e4m3fn): q = fp8(w / s), s = max|w_row| / 448.
 `linear` is bound once per (device, dtype): on the host the plain-op composition (dequantize,
 then a dense linear, saving only `q` / `scale` for the input gradient); on a GPU the
-`quant_linear` op the registry resolves (the HIP dequant-GEMM on gfx950).
-Mirrors reference `src/kohakumoss/quant/weights.py:31-140,159-190` without the ConvRot rotation
-and int8-compute variants.
+`quant_linear` op the registry resolves (the HIP dequant-GEMM on gfx950) or, for an int8 base
+with `int8_dgrad` set (int8 compute), the `int8_linear` op (activations quantized per row, int8
+MFMA GEMM). Mirrors reference `src/kohakumoss/quant/weights.py:31-140,159-202` without the
+ConvRot rotation.
 """
 
 from functools import partial
@@ -40,13 +41,17 @@ def dequantize(q: Tensor, scale: Tensor, dtype: torch.dtype) -> Tensor:
 
 
 class QuantWeight(nn.Module):
-    """BaseWeight holding `q` and `scale` as buffers (they follow `.to(device)`)."""
+    """BaseWeight holding `q` and `scale` as buffers (they follow `.to(device)`); `int8_dgrad`
+    is None (weight-only) or the input-gradient mode of int8 compute ("int8" | "16bit")."""
 
-    def __init__(self, q: Tensor, scale: Tensor, fmt: str):
+    def __init__(self, q: Tensor, scale: Tensor, fmt: str, int8_dgrad: str | None = None):
         super().__init__()
         if fmt not in FORMATS:
             raise ValueError(f"quant format {fmt!r} not in {FORMATS}")
+        if int8_dgrad is not None and fmt != "int8":
+            raise ValueError("int8 compute needs an int8 base")
         self.fmt = fmt
+        self.int8_dgrad = int8_dgrad
         self.register_buffer("q", q)
         self.register_buffer("scale", scale.float())
         self.shape = q.shape
@@ -67,6 +72,10 @@ class QuantWeight(nn.Module):
         device = self.q.device if device is None else torch.device(device)
         if device.type == "cpu":
             self._linear = _host_linear
+            return
+        if self.int8_dgrad is not None:
+            kernel = registry.resolve("int8_linear", device, dtype, group=0, dgrad=self.int8_dgrad)
+            self._linear = partial(_int8_linear, kernel)
             return
         kernel = registry.resolve("quant_linear", device, dtype, fmt=self.fmt)
         self._linear = partial(_kernel_linear, kernel)
@@ -104,3 +113,7 @@ def _host_linear(qw: QuantWeight, x: Tensor, bias: Tensor | None) -> Tensor:
 
 def _kernel_linear(kernel, qw: QuantWeight, x: Tensor, bias: Tensor | None) -> Tensor:
     return kernel(x, qw.q, qw.scale, bias, qw.fmt)
+
+
+def _int8_linear(kernel, qw: QuantWeight, x: Tensor, bias: Tensor | None) -> Tensor:
+    return kernel(x, qw.q, qw.scale, bias, 0, qw.int8_dgrad)

@@ -130,3 +130,20 @@ def test_int8_linear_leading_dims_compile_and_support():
     assert "not in" in registry.available("int8_linear", DEV, torch.bfloat16, group=0, dgrad="fp4")["hip"]
     with pytest.raises(ValueError):
         op(x.to(DEV)[..., :320], q.to(DEV)[:, :320], scale.to(DEV), None, 0, "int8")  # K % 128
+
+
+def test_quant_weight_module_runs_int8_compute():
+    from kohakumosstrainer_amd.quant.weights import QuantWeight
+
+    g = torch.Generator().manual_seed(8)
+    w = torch.randn(384, 512, generator=g) * 0.05
+    x = torch.randn(64, 512, generator=g).to(torch.bfloat16)
+    from kohakumosstrainer_amd.quant.bind import rebind_quant, set_int8_compute
+
+    base = QuantWeight.from_weight(w, "int8").to(DEV)
+    assert set_int8_compute(base, "int8") == 1
+    rebind_quant(base, DEV, torch.bfloat16)
+    y = base.linear(x.to(DEV), None)
+    assert torch.equal(y.cpu(), oi.forward(x, base.q.cpu(), base.scale.cpu(), None))
+    with pytest.raises(ValueError):
+        QuantWeight.from_weight(w, "fp8").__class__(base.q, base.scale, "fp8", int8_dgrad="int8")
