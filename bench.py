@@ -54,6 +54,14 @@ def event_ms(fn, reps: int) -> float:
     return start.elapsed_time(end) / reps
 
 
+def warm_event_ms(fn, reps: int) -> float:
+    """`event_ms` after 50 ms of the same calls."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.05:
+        fn()
+    return event_ms(fn, reps)
+
+
 def cpu_baseline(x, wq, ws, bias):
     """The oracle's eager forward (quantize, dequantize both operands, bf16 linear) on the
     first CPU_SAMPLE_ROWS rows of the same activations, all host threads, best of 3."""
@@ -84,17 +92,9 @@ def other_configs(dev, reps):
     back to back): weight-only int8 / e4m3 GEMMs, the frozen-base MXFP8 forward + input
     gradient of the adapter-training shape, and the row-recipe fp8 and int8 compute linears at
     the headline shape."""
-    import time
-
     from kohakumosstrainer_amd import native
 
-    timed_raw = event_ms
-
-    def event_ms(fn, reps):  # noqa: F811  (each measurement starts from sustained clocks)
-        t0 = time.perf_counter()
-        while time.perf_counter() - t0 < 0.05:
-            fn()
-        return timed_raw(fn, reps)
+    event_ms = warm_event_ms  # each measurement here starts from sustained clocks
 
     g = torch.Generator(device="cpu").manual_seed(0)
     out = {}

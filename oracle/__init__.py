@@ -3,7 +3,7 @@
 Everything under this directory restates, on the CPU with torch / numpy / plain C, what
 the reference's eager (torch) path computes for the quantized linear: the fp8 / MXFP8
 quantizers and dequantizers, the dequantize-then-matmul linear forward and input
-gradient, the weight-only int8 / fp8 linear, and the error statistics the reference's
+gradient, the weight-only int8 / fp8 linear, the int8 compute linear, and the error statistics the reference's
 tests judge a kernel by. Only `tests/`, `__graft_entry__.smoke()` and the
 `cpu_baseline` leg of `bench.py` may import it, and only as the checker: the shipped
 package never imports it and has no CPU fallback on a GPU.
@@ -25,6 +25,12 @@ How each function is pinned (independently of its own formula):
   linear.*                     fp64 matmul of the exactly dequantized operands
                                (tolerance, as the reference's own tests do)
   weights.quantize             np.rint half-to-even known answers, 2^-4 error bound
+  int8.quantize_rows           the reference tests' half-to-even known answers and floor
+                               scale; numpy float32 division and np.rint
+  int8.int_mm                  Python-integer matrix product
+  int8.forward / dgrad         an fp64 model of the scheme: exact agreement on inputs
+                               that quantize without error, closeness elsewhere,
+                               broken designs must fail (tests/test_oracle_int8.py)
   mxq.c (C restatement)        bit-compared against formats.quantize on random,
                                edge-case and exhaustive bf16 inputs
 
