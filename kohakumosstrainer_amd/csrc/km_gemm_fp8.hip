@@ -79,11 +79,11 @@ __device__ __forceinline__ void mfma_acc(v4f& c, const v8i& a, const v8i& b, int
 // consecutive K bytes of row l%16 in both operands, so each 16-byte half of a 128-byte-step
 // fragment (K bytes [16g, 16g+16) and [64+16g, 64+16g+16)) feeds one instruction: two of them
 // cover the step, in a K order that is the same for both operands.
-__device__ __forceinline__ void mfma_i8_acc(v4f& c, const v8i& a, const v8i& b) {
-  const v4i a_lo = __builtin_shufflevector(a, a, 0, 1, 2, 3), b_lo = __builtin_shufflevector(b, b, 0, 1, 2, 3);
-  const v4i a_hi = __builtin_shufflevector(a, a, 4, 5, 6, 7), b_hi = __builtin_shufflevector(b, b, 4, 5, 6, 7);
-  asm("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a_lo), "v"(b_lo));
-  asm("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a_hi), "v"(b_hi));
+template <bool HI>
+__device__ __forceinline__ void mfma_i8_half(v4f& c, const v8i& a, const v8i& b) {
+  const v4i ah = HI ? __builtin_shufflevector(a, a, 4, 5, 6, 7) : __builtin_shufflevector(a, a, 0, 1, 2, 3);
+  const v4i bh = HI ? __builtin_shufflevector(b, b, 4, 5, 6, 7) : __builtin_shufflevector(b, b, 0, 1, 2, 3);
+  asm("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(ah), "v"(bh));
 }
 
 // A1: one A buffer instead of two (the A slab of step k+1 is requested at the top of step k,
@@ -282,9 +282,18 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
       static_for<TM>([&](auto j_tag) __attribute__((always_inline)) {
         constexpr int j = decltype(j_tag)::value;
         constexpr int q = t * TM + j;  // position in the step's MFMA sequence
-        if constexpr (I8)
-          mfma_i8_acc(acc[t][j], wcur, xf[j]);
-        else if constexpr (SCALE_KM)
+        if constexpr (I8) {
+          // two tiles per pair of slots, low halves then high halves: the two instructions that
+          // add into one accumulator are two instructions apart instead of back to back
+          static_assert(TM % 2 == 0, "int8 tiles are issued in pairs");
+          if constexpr ((j & 1) == 0) {
+            mfma_i8_half<false>(acc[t][j], wcur, xf[j]);
+            mfma_i8_half<false>(acc[t][j + 1], wcur, xf[j + 1]);
+          } else {
+            mfma_i8_half<true>(acc[t][j - 1], wcur, xf[j - 1]);
+            mfma_i8_half<true>(acc[t][j], wcur, xf[j]);
+          }
+        } else if constexpr (SCALE_KM)
           mfma_acc<t, j>(acc[t][j], wcur, xf[j], wscale[P][(t >> 2) % WS], xscale[P][(j >> 2) % XS]);
         else
           mfma_acc<0, 0>(acc[t][j], wcur, xf[j], wscale[P][t % WS], xscale[P][j % XS]);
