@@ -135,6 +135,16 @@ int km_wo_gemm_dgrad(const void *dy, const void *q, const float *scale, void *dx
                      void *q_t_workspace, int64_t M, int64_t N, int64_t K, int q_format, int dtype,
                      int config, void *stream);
 
+/* Group Hadamard rotation (ConvRot): y[r, :] = x[r, :] . blockdiag(H_group), H_group the normalised
+ * Kronecker power of H4 = [[1,1,1,-1],[1,1,-1,1],[1,-1,1,1],[-1,1,1,1]] (symmetric, its own
+ * inverse), group in {4, 16, 64, 256, 1024} dividing cols; x and y [rows, cols] contiguous,
+ * 16-byte aligned, dtype KM_BF16 / KM_F16. fp32 4-point butterflies in the reference's stage
+ * order, one scaling by 1/sqrt(group), one rounding. Replaces the Triton rotation
+ * (backends/triton/hadamard.py:28-105) and hadamard.group_hadamard_eager
+ * (src/kohakumoss_kernels/hadamard.py:71-101). */
+int km_group_hadamard(const void *x, int64_t rows, int64_t cols, int dtype, int group, void *y,
+                      void *stream);
+
 /* Tile configurations per kernel, for the host-side tuning table (the reference enumerates its
  * Triton tiles in backends/triton/fp8/linear.py:39-75 and backends/triton/quant.py:132-141). */
 int km_num_configs(int kernel);

@@ -38,6 +38,7 @@ EXPORTS = (
     "km_gemm_i8_rows",
     "km_wo_gemm_fwd",
     "km_wo_gemm_dgrad",
+    "km_group_hadamard",
     "km_num_configs",
     "km_config_desc",
 )
@@ -71,6 +72,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.km_gemm_i8_rows.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_wo_gemm_fwd.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_wo_gemm_dgrad.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
+    lib.km_group_hadamard.argtypes = [p, i64, i64, i32, i32, p, p]
     lib.km_num_configs.argtypes = [i32]
     lib.km_config_desc.argtypes = [i32, i32, c.c_char_p, i32]
     for name in EXPORTS:
@@ -240,6 +242,18 @@ def quant_rows_i8(x: Tensor, col_scale: Tensor | None = None) -> tuple[Tensor, T
     with torch.cuda.device(x.device):
         _check(load().km_quant_rows_i8(x.data_ptr(), rows, k, x.stride(0), x.stride(1), _dtype_code(x.dtype), None if col_scale is None else col_scale.data_ptr(), q.data_ptr(), s.data_ptr(), _stream(x)))
     return q, s
+
+
+def group_hadamard(x: Tensor, group: int) -> Tensor:
+    """`x [rows, K]` (bf16 / fp16) times blockdiag(H_group) over K, a new contiguous tensor."""
+    if x.dim() != 2:
+        raise ValueError(f"rotation operand must be 2-D, got {tuple(x.shape)}")
+    _on_gpu(x)
+    x = x.contiguous()
+    y = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        _check(load().km_group_hadamard(x.data_ptr(), x.shape[0], x.shape[1], _dtype_code(x.dtype), int(group), y.data_ptr(), _stream(x)))
+    return y
 
 
 # ---- GEMMs --------------------------------------------------------------------------------
