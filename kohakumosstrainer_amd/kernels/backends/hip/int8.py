@@ -2,14 +2,15 @@
 int32 MFMA with both scales and the bias applied to the accumulator in the eager path's order of
 roundings (outputs equal the eager reference bit for bit), and the two input-gradient modes.
 Host-side counterpart of reference `backends/triton/int8.py` (launchers :234-270, registration
-:273-281). The int8 input gradient contracts over N, so it reads a `[K, N]` copy of the codes,
+:273-281). A rotated base (`group` > 0) gets one pass of the HIP butterfly kernel over x before
+the quantizer and one over dx. The int8 input gradient contracts over N, so it reads a `[K, N]` copy of the codes,
 made per call as the reference makes its column-major copy (`int8/formats.py:55-58`).
 """
 
 from kohakumosstrainer_amd import native
 from kohakumosstrainer_amd.kernels import registry, tuning
 from kohakumosstrainer_amd.kernels.constraints import requires
-from kohakumosstrainer_amd.kernels.errors import BackendUnavailable
+from kohakumosstrainer_amd.kernels.hadamard import rotate_2d
 from kohakumosstrainer_amd.kernels.int8.op import int8_supported, make_int8_linear, register_launchers
 from kohakumosstrainer_amd.kernels.tuning import pow2
 
@@ -25,9 +26,7 @@ def candidates(m: int) -> list[dict]:
     return sorted(fits, key=lambda c: -(c["bm"] * c["bn"]) if m >= 1024 else c["bm"])
 
 
-def _check(kind, contraction, group):
-    if group:
-        raise BackendUnavailable(f"int8_{kind}", {"hip": f"rotation group {group} is not built for gfx950"}, persist=False)
+def _check(kind, contraction):
     if contraction % ALIGN_K:
         raise ValueError(f"int8_{kind}: contraction length {contraction} must be a multiple of {ALIGN_K}")
 
@@ -46,9 +45,9 @@ def _pick(kernel, kind, m, n, k, a, bias, launch, in_backward):
 def fwd(x, q, scale, bias, group):
     m, k = x.shape
     n = q.shape[0]
-    _check("fwd", k, group)
+    _check("fwd", k)
     q, scale = q.contiguous(), scale.float().contiguous()
-    xq, xs = native.quant_rows_i8(x)
+    xq, xs = native.quant_rows_i8(rotate_2d(x, group) if group else x)
     cfg = _pick("int8_fwd", "fwd", m, n, k, x, bias, lambda c: lambda: native.gemm_i8_rows(xq, xs, q, scale, bias, x.dtype, c["id"]), False)
     return native.gemm_i8_rows(xq, xs, q, scale, bias, x.dtype, cfg["id"])
 
@@ -57,13 +56,14 @@ def dgrad(dy, q, scale, group, mode):
     m, n = dy.shape
     k = q.shape[1]
     if mode == "16bit":
-        _check("dgrad", 0, group)
-        return native.wo_gemm_dgrad(dy, q.contiguous(), scale, 0)
-    _check("dgrad", n, group)
+        dx = native.wo_gemm_dgrad(dy, q.contiguous(), scale, 0)
+        return rotate_2d(dx, group) if group else dx
+    _check("dgrad", n)
     gq, gs = native.quant_rows_i8(dy, scale)
     q_t = q.t().contiguous()
     cfg = _pick("int8_dgrad", "dgrad", m, k, n, dy, None, lambda c: lambda: native.gemm_i8_rows(gq, gs, q_t, None, None, dy.dtype, c["id"]), True)
-    return native.gemm_i8_rows(gq, gs, q_t, None, None, dy.dtype, cfg["id"])
+    dx = native.gemm_i8_rows(gq, gs, q_t, None, None, dy.dtype, cfg["id"])
+    return rotate_2d(dx, group) if group else dx
 
 
 register_launchers("hip", fwd, dgrad)

@@ -225,7 +225,7 @@ def load_backends() -> None:
         if _loaded:
             return
         _loaded.append(True)
-        for mod in ("fp8.op", "fp8.train", "quant", "int8.op"):
+        for mod in ("fp8.op", "fp8.train", "quant", "hadamard", "rotated", "int8.op"):
             importlib.import_module(f"kohakumosstrainer_amd.kernels.{mod}")
         try:
             importlib.import_module("kohakumosstrainer_amd.kernels.backends.hip")

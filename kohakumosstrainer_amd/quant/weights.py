@@ -6,8 +6,9 @@ fp8 (e4m3fn): q = fp8(w / s), s = max|w_row| / 448.
 then a dense linear, saving only `q` / `scale` for the input gradient); on a GPU the
 `quant_linear` op the registry resolves (the HIP dequant-GEMM on gfx950) or, for an int8 base
 with `int8_dgrad` set (int8 compute), the `int8_linear` op (activations quantized per row, int8
-MFMA GEMM). Mirrors reference `src/kohakumoss/quant/weights.py:31-140,159-202` without the
-ConvRot rotation.
+MFMA GEMM). `rotation` > 0 marks a ConvRot base: the stored codes are those of W R with
+R = blockdiag(H_rotation) over K, and the linear rotates x first (`quant_linear_rotated`, or the
+`group` of `int8_linear`). Mirrors reference `src/kohakumoss/quant/weights.py:31-140,159-202`.
 """
 
 from functools import partial
@@ -44,13 +45,14 @@ class QuantWeight(nn.Module):
     """BaseWeight holding `q` and `scale` as buffers (they follow `.to(device)`); `int8_dgrad`
     is None (weight-only) or the input-gradient mode of int8 compute ("int8" | "16bit")."""
 
-    def __init__(self, q: Tensor, scale: Tensor, fmt: str, int8_dgrad: str | None = None):
+    def __init__(self, q: Tensor, scale: Tensor, fmt: str, rotation: int = 0, int8_dgrad: str | None = None):
         super().__init__()
         if fmt not in FORMATS:
             raise ValueError(f"quant format {fmt!r} not in {FORMATS}")
         if int8_dgrad is not None and fmt != "int8":
             raise ValueError("int8 compute needs an int8 base")
         self.fmt = fmt
+        self.rotation = int(rotation)
         self.int8_dgrad = int8_dgrad
         self.register_buffer("q", q)
         self.register_buffer("scale", scale.float())
@@ -62,7 +64,12 @@ class QuantWeight(nn.Module):
         return cls(*quantize(w, fmt), fmt)
 
     def weight(self, dtype: torch.dtype) -> Tensor:
-        return dequantize(self.q, self.scale, dtype)
+        """W in `dtype` (the rotation undone: W = (q * s) R, R its own inverse)."""
+        if not self.rotation:
+            return dequantize(self.q, self.scale, dtype)
+        from kohakumosstrainer_amd.kernels.hadamard import group_hadamard_eager
+
+        return group_hadamard_eager(dequantize(self.q, self.scale, torch.float32), self.rotation).to(dtype)
 
     def materialize(self) -> Tensor:
         return self.weight(torch.float32)
@@ -74,8 +81,12 @@ class QuantWeight(nn.Module):
             self._linear = _host_linear
             return
         if self.int8_dgrad is not None:
-            kernel = registry.resolve("int8_linear", device, dtype, group=0, dgrad=self.int8_dgrad)
+            kernel = registry.resolve("int8_linear", device, dtype, group=self.rotation, dgrad=self.int8_dgrad)
             self._linear = partial(_int8_linear, kernel)
+            return
+        if self.rotation:
+            kernel = registry.resolve("quant_linear_rotated", device, dtype, fmt=self.fmt, group=self.rotation)
+            self._linear = partial(_rotated_linear, kernel)
             return
         kernel = registry.resolve("quant_linear", device, dtype, fmt=self.fmt)
         self._linear = partial(_kernel_linear, kernel)
@@ -106,6 +117,10 @@ class _HostLinear(torch.autograd.Function):
 
 
 def _host_linear(qw: QuantWeight, x: Tensor, bias: Tensor | None) -> Tensor:
+    if qw.rotation:
+        from kohakumosstrainer_amd.kernels.rotated import quant_linear_rotated_eager
+
+        return quant_linear_rotated_eager(x, qw.q, qw.scale, bias, qw.fmt, qw.rotation)
     lead = x.shape[:-1]
     y = _HostLinear.apply(x.reshape(-1, x.shape[-1]), qw.q, qw.scale, bias)
     return y.reshape(*lead, qw.q.shape[0])
@@ -115,5 +130,9 @@ def _kernel_linear(kernel, qw: QuantWeight, x: Tensor, bias: Tensor | None) -> T
     return kernel(x, qw.q, qw.scale, bias, qw.fmt)
 
 
+def _rotated_linear(kernel, qw: QuantWeight, x: Tensor, bias: Tensor | None) -> Tensor:
+    return kernel(x, qw.q, qw.scale, bias, qw.fmt, qw.rotation)
+
+
 def _int8_linear(kernel, qw: QuantWeight, x: Tensor, bias: Tensor | None) -> Tensor:
-    return kernel(x, qw.q, qw.scale, bias, 0, qw.int8_dgrad)
+    return kernel(x, qw.q, qw.scale, bias, qw.rotation, qw.int8_dgrad)

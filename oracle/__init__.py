@@ -31,6 +31,8 @@ How each function is pinned (independently of its own formula):
   int8.forward / dgrad         an fp64 model of the scheme: exact agreement on inputs
                                that quantize without error, closeness elsewhere,
                                broken designs must fail (tests/test_oracle_int8.py)
+  hadamard.*                   fp64 torch.kron construction, H H = I, exact equality on
+                               integer inputs (tests/test_oracle_hadamard.py)
   mxq.c (C restatement)        bit-compared against formats.quantize on random,
                                edge-case and exhaustive bf16 inputs
 

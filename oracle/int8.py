@@ -3,8 +3,9 @@
 per-row quantizer   reference `src/kohakumoss_kernels/int8/formats.py:21-38`
 int8 GEMM           reference `int8/formats.py:41-52` (`torch._int_mm`, int32 accumulation; here
                     the fp64 matmul of the codes, exact because |acc| <= K * 127^2 < 2^53)
-forward / dgrad     reference `src/kohakumoss_kernels/int8/op.py:40-60` with `group` 0 (no
-                    rotation: ConvRot is outside this path)
+forward / dgrad     reference `src/kohakumoss_kernels/int8/op.py:40-60`; `group` > 0 rotates x
+                    before the quantizer and dx afterwards (`oracle/hadamard.py`; `rotation`
+                    picks the reference's eager form or its kernels' butterfly form)
 
 Pinned by `tests/test_oracle_int8.py`: the reference's half-to-even known answers and floor
 scale (`tests/kernels/quant/test_int8_linear.py:142-148`), a definition-level numpy restatement,
@@ -15,6 +16,8 @@ exact agreement with an fp64 model of the scheme on inputs that quantize without
 
 import torch
 from torch import Tensor
+
+from oracle import hadamard
 
 INT8_MAX = 127.0
 AMAX_FLOOR = 1e-12
@@ -49,22 +52,28 @@ def dequantize_weight(q: Tensor, scale: Tensor, dtype: torch.dtype) -> Tensor:
     return (q.to(torch.float32) * scale.to(torch.float32)[:, None]).to(dtype)
 
 
-def forward(x: Tensor, q: Tensor, scale: Tensor, bias: Tensor | None) -> Tensor:
-    """`(int32(Q(x) q^T) * s_x) * s_w (+ bias)` in fp32, each operation rounded on its own,
-    rounded once to x's dtype."""
-    xq, xs = quantize_rows(x)
+def _rotate(t: Tensor, group: int, rotation: str) -> Tensor:
+    if not group:
+        return t
+    return hadamard.butterflies(t, group) if rotation == "butterflies" else hadamard.rotate(t, group)
+
+
+def forward(x: Tensor, q: Tensor, scale: Tensor, bias: Tensor | None, group: int = 0, rotation: str = "eager") -> Tensor:
+    """`(int32(Q(x R) q^T) * s_x) * s_w (+ bias)` in fp32, each operation rounded on its own,
+    rounded once to x's dtype; x R is rounded to x's dtype before it is quantized."""
+    xq, xs = quantize_rows(_rotate(x, group, rotation))
     y = int_mm(xq, q.t()).to(torch.float32) * xs[:, None] * scale.to(torch.float32)[None, :]
     if bias is not None:
         y = y + bias.to(torch.float32)
     return y.to(x.dtype)
 
 
-def dgrad(dy: Tensor, q: Tensor, scale: Tensor, mode: str) -> Tensor:
+def dgrad(dy: Tensor, q: Tensor, scale: Tensor, mode: str, group: int = 0, rotation: str = "eager") -> Tensor:
     """int8: `Q(dy * scale) q` (int32) times dy's row scales; 16bit: `dy (q * scale)`, the
-    weight-only input gradient."""
+    weight-only input gradient; both rotated back when the base is a rotated one."""
     if mode not in DGRAD:
         raise ValueError(f"int8 dgrad {mode!r} not in {DGRAD}")
     if mode == "16bit":
-        return dy @ dequantize_weight(q, scale, dy.dtype)
+        return _rotate(dy @ dequantize_weight(q, scale, dy.dtype), group, rotation)
     gq, gs = quantize_rows(dy, scale)
-    return (int_mm(gq, q).to(torch.float32) * gs[:, None]).to(dy.dtype)
+    return _rotate((int_mm(gq, q).to(torch.float32) * gs[:, None]).to(dy.dtype), group, rotation)

@@ -126,7 +126,8 @@ def test_int8_linear_leading_dims_compile_and_support():
     assert torch.equal(y.cpu().reshape(128, 256), oi.forward(x.reshape(128, 512), q, scale, None))
     compiled = torch.compile(lambda t: op(t, q.to(DEV), scale.to(DEV), None, 0, "int8"), fullgraph=True)
     assert torch.equal(compiled(x.to(DEV)), y)
-    assert "not built" in registry.available("int8_linear", DEV, torch.bfloat16, group=256, dgrad="int8")["hip"]
+    assert registry.available("int8_linear", DEV, torch.bfloat16, group=256, dgrad="int8")["hip"] is None
+    assert "power of 4" in registry.available("int8_linear", DEV, torch.bfloat16, group=8, dgrad="int8")["hip"]
     assert "not in" in registry.available("int8_linear", DEV, torch.bfloat16, group=0, dgrad="fp4")["hip"]
     with pytest.raises(ValueError):
         op(x.to(DEV)[..., :320], q.to(DEV)[:, :320], scale.to(DEV), None, 0, "int8")  # K % 128
@@ -147,3 +148,68 @@ def test_quant_weight_module_runs_int8_compute():
     assert torch.equal(y.cpu(), oi.forward(x, base.q.cpu(), base.scale.cpu(), None))
     with pytest.raises(ValueError):
         QuantWeight.from_weight(w, "fp8").__class__(base.q, base.scale, "fp8", int8_dgrad="int8")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("group", (64, 256))
+def test_rotated_int8_linear(dtype, group):
+    """A ConvRot base: x is rotated by the HIP butterfly kernel before the quantizer and dx after
+    the GEMM. Against the oracle with the butterfly form of the rotation the result is equal bit
+    for bit; against the reference's eager form (a 16-bit matmul with H, whose fp32 sums round
+    in another order) and the fp64 model it is close."""
+    from oracle import hadamard as oh
+
+    m, n, k = 200, 384, 1024
+    g = torch.Generator().manual_seed(group)
+    q, scale = weight(n, k, g)
+    x = torch.randn(m, k, generator=g).to(dtype)
+    bias = (torch.randn(n, generator=g) * 0.1).to(dtype)
+    dy = torch.randn(m, n, generator=g).to(dtype)
+    for mode in oi.DGRAD:
+        op = registry.resolve("int8_linear", DEV, dtype, group=group, dgrad=mode)
+        assert op.backend == "hip"
+        xd = x.to(DEV).requires_grad_(True)
+        y = op(xd, q.to(DEV), scale.to(DEV), bias.to(DEV), group, mode)
+        y.backward(dy.to(DEV))
+        assert torch.equal(y.detach().cpu(), oi.forward(x, q, scale, bias, group, "butterflies"))
+        eager = oi.forward(x, q, scale, bias, group)
+        h = oh.matrix(group).double()
+        xr = (x.double().reshape(-1, group) @ h).reshape(m, k)
+        s64 = xr.abs().amax(1).clamp_min(1e-12) / 127.0
+        exact = (torch.round(xr / s64[:, None]).clamp(-127, 127) @ q.double().T) * s64[:, None] * scale.double()[None, :] + bias.double()
+        oracle_stats.assert_no_regression(y.detach().cpu(), eager, exact, name=f"rotated fwd g{group}")
+        want_dx = oi.dgrad(dy, q, scale, mode, group, "butterflies")
+        if mode == "int8":
+            assert torch.equal(xd.grad.cpu(), want_dx)
+        else:
+            exact_dx = ((dy.double() @ (q.double() * scale.double()[:, None])).reshape(-1, group) @ h).reshape(m, k)
+            oracle_stats.assert_no_regression(xd.grad.cpu(), oi.dgrad(dy, q, scale, mode, group), exact_dx, name="rotated 16bit dgrad")
+
+
+def test_rotated_weight_only_linear_and_module():
+    from kohakumosstrainer_amd.quant.weights import QuantWeight
+    from oracle import hadamard as oh
+    from oracle import linear as ol
+
+    g = torch.Generator().manual_seed(12)
+    m, n, k, group = 130, 256, 768, 256
+    q, scale = weight(n, k, g)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    bias = (torch.randn(n, generator=g) * 0.1).to(torch.bfloat16)
+    dy = torch.randn(m, n, generator=g).to(torch.bfloat16)
+    op = registry.resolve("quant_linear_rotated", DEV, torch.bfloat16, fmt="int8", group=group)
+    assert op.backend == "hip"
+    xd = x.to(DEV).requires_grad_(True)
+    y = op(xd, q.to(DEV), scale.to(DEV), bias.to(DEV), "int8", group)
+    y.backward(dy.to(DEV))
+    h = oh.matrix(group).double()
+    w64 = q.double() * scale.double()[:, None]
+    exact = (x.double().reshape(-1, group) @ h).reshape(m, k) @ w64.T + bias.double()
+    eager = ol.wo_forward(oh.rotate(x, group), q, scale, bias)
+    oracle_stats.assert_no_regression(y.detach().cpu(), eager, exact, name="rotated weight-only fwd")
+    exact_dx = ((dy.double() @ w64).reshape(-1, group) @ h).reshape(m, k)
+    oracle_stats.assert_no_regression(xd.grad.cpu(), oh.rotate(ol.wo_dgrad(dy, q, scale), group), exact_dx, name="rotated weight-only dgrad")
+    base = QuantWeight(q, scale, "int8", rotation=group).to(DEV)
+    base.bind(torch.bfloat16)
+    assert torch.equal(base.linear(x.to(DEV), bias.to(DEV)), y.detach())
+    torch.testing.assert_close(base.weight(torch.float32).cpu().double(), (w64.reshape(-1, group) @ h).reshape(n, k), rtol=1e-5, atol=1e-6)

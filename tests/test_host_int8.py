@@ -57,11 +57,50 @@ def test_eager_op_matches_oracle_and_autograd_contract(mode):
     assert torch.equal(y3[0], oi.forward(x, q, scale, None))
 
 
-def test_support_check_and_rotation_refused():
+def test_support_check():
     registry.load_backends()
     assert registry.available("int8_linear", "cpu", torch.bfloat16, group=0, dgrad="int8")["eager"] is None
-    assert "not built" in registry.available("int8_linear", "cpu", torch.bfloat16, group=256, dgrad="int8")["eager"]
+    assert registry.available("int8_linear", "cpu", torch.bfloat16, group=256, dgrad="int8")["eager"] is None
+    assert "power of 4" in registry.available("int8_linear", "cpu", torch.bfloat16, group=8, dgrad="int8")["eager"]
     assert "not in" in registry.available("int8_linear", "cpu", torch.bfloat16, group=0, dgrad="fp4")["eager"]
-    x, q, scale, bias, dy = problem(4, 8, 16)
+    x, q, scale, bias, dy = problem(4, 8, 24)
     with pytest.raises(ValueError):
-        int8_op.fwd_reference(x, q, scale, bias, 64)
+        int8_op.fwd_reference(x, q, scale, bias, 16)  # 24 % 16
+
+
+@pytest.mark.parametrize("mode", int8_op.DGRAD)
+@pytest.mark.parametrize("dtype", (torch.float32, torch.bfloat16))
+def test_rotated_base_matches_oracle(mode, dtype):
+    x, q, scale, bias, dy = problem(9, 32, 128, dtype, seed=2)
+    op = registry.resolve("int8_linear", "cpu", dtype, group=64, dgrad=mode)
+    xa = x.clone().requires_grad_(True)
+    y = op(xa, q, scale, bias, 64, mode)
+    assert torch.equal(y, oi.forward(x, q, scale, bias, 64))
+    y.backward(dy)
+    assert torch.equal(xa.grad, oi.dgrad(dy, q, scale, mode, 64))
+
+
+def test_rotation_and_rotated_weight_only_on_the_host():
+    from kohakumosstrainer_amd.kernels import hadamard
+    from oracle import hadamard as oh
+    from oracle import linear as ol
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(5, 2, 128, generator=g)
+    for dt in (torch.float32, torch.bfloat16):
+        xa = x.to(dt).detach().clone().requires_grad_(True)
+        y = hadamard.group_hadamard(xa, 64)
+        assert torch.equal(y, oh.rotate(x.to(dt), 64))
+        y.backward(torch.ones_like(y))
+        assert torch.equal(xa.grad, oh.rotate(torch.ones_like(y), 64))
+    assert torch.equal(hadamard.hadamard_matrix(16), oh.matrix(16))
+    with pytest.raises(ValueError):
+        hadamard.group_hadamard(x, 48)
+    xq, q, scale, bias, dy = problem(9, 32, 128, torch.bfloat16, seed=4)
+    op = registry.resolve("quant_linear_rotated", "cpu", torch.bfloat16, fmt="int8", group=64)
+    assert op.backend == "eager"
+    xa = xq.clone().requires_grad_(True)
+    y = op(xa, q, scale, bias, "int8", 64)
+    assert torch.equal(y, ol.wo_forward(oh.rotate(xq, 64), q, scale, bias))
+    y.backward(dy)
+    assert torch.equal(xa.grad, oh.rotate(ol.wo_dgrad(dy, q, scale), 64))

@@ -133,3 +133,24 @@ def test_argument_errors():
         oi.quantize_rows(torch.zeros(4))
     with pytest.raises(ValueError):
         oi.dgrad(torch.zeros(2, 4), torch.zeros(4, 8, dtype=torch.int8), torch.ones(4), "fp4")
+
+
+@pytest.mark.parametrize("group", (16, 64))
+def test_rotated_forward_equals_the_fp64_model_on_the_grid(group):
+    """x chosen so that x R is exactly codes / 64 with a 127 per row (R is its own inverse and
+    the integers keep every butterfly exact): the rotated forward must equal the fp64 model of
+    'rotate, quantize, multiply' and differ from the unrotated one."""
+    from oracle import hadamard as oh
+
+    q, scale, g = weight(128, 256, seed=5)
+    bias = torch.randn(128, generator=g) * 0.1
+    codes = on_grid(33, 256, g)
+    h = oh.matrix(group).double()
+    x = (codes.double().reshape(-1, group) @ h).reshape(codes.shape).float()
+    assert torch.equal((x.double().reshape(-1, group) @ h).reshape(codes.shape).float(), codes)
+    y = oi.forward(x, q, scale, bias, group)
+    torch.testing.assert_close(y.double(), model64(codes, q, scale, bias), rtol=1e-5, atol=1e-5)
+    must_fail(lambda: torch.testing.assert_close(oi.forward(x, q, scale, bias).double(), model64(codes, q, scale, bias), rtol=1e-3, atol=1e-3), "no rotation")
+    dy = torch.randn(33, 128, generator=g)
+    want = (dx64(dy, q, scale, "int8").reshape(-1, group) @ h).reshape(33, 256)
+    torch.testing.assert_close(oi.dgrad(dy, q, scale, "int8", group).double(), want, rtol=1e-3, atol=1e-3)
