@@ -90,8 +90,8 @@ def cpu_baseline(x, wq, ws, bias):
 def other_configs(dev, reps):
     """Device time of the other kernels of the path at their benchmark shapes (event-timed,
     back to back): weight-only int8 / e4m3 GEMMs, the frozen-base MXFP8 forward + input
-    gradient of the adapter-training shape, and the row-recipe fp8 and int8 compute linears at
-    the headline shape."""
+    gradient of the adapter-training shape, and the row-recipe, block-recipe fp8 and int8 compute
+    linears at the headline shape."""
     from kohakumosstrainer_amd import native
 
     event_ms = warm_event_ms  # each measurement here starts from sustained clocks
@@ -165,6 +165,27 @@ def other_configs(dev, reps):
     flop = 2 * m * n * k
     out["row_recipe_M16384_K3072_N9216"] = {
         "quant_rows_us": qt * 1e3, "quant_rows_GBps": (m * k * 3 + m * 4) / qt / 1e6, "hbm_peak_GBps": HBM_PEAK_GBS,
+        "gemm_ms": gt, "gemm_TFLOPs": flop / gt / 1e9, "step_ms": st, "step_TFLOPs": flop / st / 1e9, "peak_TFLOPs": FP8_PEAK_TFLOPS,
+    }
+    # the block recipe (fp32 scales per row x 128 columns / per 128 x 128 weight block), same shape
+    wbq, wbs = native.quant_blocks(w, "weight")
+    xbq, xbs = native.quant_blocks(x, "act")
+    bsbuf = torch.empty(m, k // 128, dtype=torch.float32, device=dev)
+
+    def quant_blocks_only():
+        lib.km_quant_blocks(x.data_ptr(), m, k, k, 1, native.KM_BF16, native.ROLE_ACT, qbuf.data_ptr(), bsbuf.data_ptr(), stream)
+
+    def block_step():
+        aq, sa = native.quant_blocks(x, "act")
+        return native.gemm_fp8_blocks(aq, sa, wbq, wbs, bias, torch.bfloat16, 0)
+
+    quant_blocks_only()
+    block_step()
+    qt = event_ms(quant_blocks_only, reps)
+    gt = event_ms(lambda: native.gemm_fp8_blocks(xbq, xbs, wbq, wbs, bias, torch.bfloat16, 0), reps)
+    st = event_ms(block_step, reps)
+    out["block_recipe_M16384_K3072_N9216"] = {
+        "quant_blocks_us": qt * 1e3, "quant_blocks_GBps": (m * k * 3 + m * (k // 128) * 4) / qt / 1e6, "hbm_peak_GBps": HBM_PEAK_GBS,
         "gemm_ms": gt, "gemm_TFLOPs": flop / gt / 1e9, "step_ms": st, "step_TFLOPs": flop / st / 1e9, "peak_TFLOPs": FP8_PEAK_TFLOPS,
     }
     # int8 compute linear (per-row int8 activations, int8 MFMA GEMM, int32 accumulation), same shape

@@ -27,6 +27,7 @@ extern "C" int km_num_configs(int kernel) {
     case KM_KERNEL_GEMM_FP8: return km::gemm_num_configs();
     case KM_KERNEL_WO_FWD:
     case KM_KERNEL_WO_DGRAD: return km::wo_num_configs();
+    case KM_KERNEL_GEMM_BLOCKS: return km::blocks_gemm_num_configs();
   }
   return km_fail(KM_ERR_ARG, "km_num_configs: unknown kernel");
 }
@@ -38,6 +39,7 @@ extern "C" int km_config_desc(int kernel, int config, char* buf, int len) {
     case KM_KERNEL_GEMM_FP8: return km::gemm_config_desc(config, buf, len);
     case KM_KERNEL_WO_FWD:
     case KM_KERNEL_WO_DGRAD: return km::wo_config_desc(config, buf, len);
+    case KM_KERNEL_GEMM_BLOCKS: return km::blocks_gemm_config_desc(config, buf, len);
   }
   return km_fail(KM_ERR_ARG, "km_config_desc: unknown kernel");
 }

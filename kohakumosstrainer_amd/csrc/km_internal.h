@@ -13,4 +13,6 @@ int gemm_num_configs();
 int gemm_config_desc(int config, char* buf, int len);
 int wo_num_configs();
 int wo_config_desc(int config, char* buf, int len);
+int blocks_gemm_num_configs();
+int blocks_gemm_config_desc(int config, char* buf, int len);
 }  // namespace km

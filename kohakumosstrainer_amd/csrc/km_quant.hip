@@ -742,6 +742,133 @@ __global__ __launch_bounds__(256) void quant_i8_rows_generic(const uint16_t* __r
   }
 }
 
+// ---- block recipe: fp32 scales per 128 columns (activations) or per 128 x 128 block (weights) ----
+// s = max(amax, 1e-12) / 448 and q = e4m3(clamp(x / s)) as in the per-row recipe, over smaller
+// groups (reference src/kohakumoss_kernels/fp8/formats.py:83-93).
+
+// max over the 16 lanes of a DPP row, in every lane of the row
+__device__ __forceinline__ uint32_t row16_max(uint32_t v) {
+  v = quad_max(v);
+  uint32_t o = (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x124, 0xF, 0xF, true);  // row_ror:4
+  v = v > o ? v : o;
+  o = (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x128, 0xF, 0xF, true);  // row_ror:8
+  return v > o ? v : o;
+}
+
+// Activations, unit-stride rows: lane = 8 consecutive elements, 16 lanes = one block of 128.
+// q and the scales [rows, cols/128] are contiguous, so both are indexed by the flat group number.
+template <int DT>
+__global__ __launch_bounds__(kRowsThreads) void quant_fp8_blocks_act(const uint16_t* __restrict__ x, int64_t ld, uint32_t groups_per_row,
+                                                                     uint64_t ngroups, uint8_t* __restrict__ q, float* __restrict__ scale) {
+  saturating_conversions();
+  const uint64_t base = (uint64_t)blockIdx.x * (kRowsThreads * kRowsUnroll) + threadIdx.x;
+  const bool dense = ld == (int64_t)groups_per_row * 8;
+  uint4 raw[kRowsUnroll];
+#pragma unroll
+  for (int u = 0; u < kRowsUnroll; ++u) {
+    const uint64_t g = base + (uint64_t)u * kRowsThreads;
+    raw[u] = make_uint4(0, 0, 0, 0);
+    if (g < ngroups) {
+      uint64_t off;
+      if (dense) {
+        off = g * 8;
+      } else {
+        const uint64_t row = g / groups_per_row;
+        off = row * (uint64_t)ld + (g - row * groups_per_row) * 8;
+      }
+      raw[u] = *reinterpret_cast<const uint4*>(x + off);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kRowsUnroll; ++u) {
+    const uint64_t g = base + (uint64_t)u * kRowsThreads;
+    const uint32_t m16 = row16_max(amax16x8(raw[u]));
+    const float s = scale_of_amax16<DT>(m16);
+    const float rcp = __fdiv_rn(1.0f, s);
+    const uint2 codes = divided_codes8<DT>(raw[u], s, rcp, m16 < inf16<DT>(), m16 > inf16<DT>());
+    if (g < ngroups) {
+      *reinterpret_cast<uint2*>(q + g * 8) = codes;
+      if ((threadIdx.x & 15) == 0) scale[g >> 4] = s;
+    }
+  }
+}
+
+// Weights, unit-stride rows: a workgroup owns one 128 x 128 block, held in registers (eight
+// 128-bit loads per lane) between the amax pass and the conversion. Rows past the end count as zeros.
+template <int DT>
+__global__ __launch_bounds__(256) void quant_fp8_blocks_weight(const uint16_t* __restrict__ x, int64_t ld, int64_t rows, int64_t cols,
+                                                               uint8_t* __restrict__ q, float* __restrict__ scale) {
+  saturating_conversions();
+  __shared__ uint32_t wave_amax[4];
+  const int64_t r0 = (int64_t)blockIdx.y * 128, c0 = (int64_t)blockIdx.x * 128;
+  const int chunk = threadIdx.x & 15, rsub = threadIdx.x >> 4;
+  uint4 raw[8];
+  uint32_t m16 = 0;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int64_t r = r0 + rsub + 16 * u;
+    raw[u] = r < rows ? *reinterpret_cast<const uint4*>(x + r * ld + c0 + chunk * 8) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const uint32_t a = amax16x8(raw[u]);
+    m16 = a > m16 ? a : m16;
+  }
+  m16 = wave_max(m16);
+  if ((threadIdx.x & 63) == 0) wave_amax[threadIdx.x >> 6] = m16;
+  __syncthreads();
+  m16 = max(max(wave_amax[0], wave_amax[1]), max(wave_amax[2], wave_amax[3]));
+  const float s = scale_of_amax16<DT>(m16);
+  const float rcp = __fdiv_rn(1.0f, s);
+  if (threadIdx.x == 0) scale[(int64_t)blockIdx.y * gridDim.x + blockIdx.x] = s;
+  const bool finite = m16 < inf16<DT>(), nan_block = m16 > inf16<DT>();
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int64_t r = r0 + rsub + 16 * u;
+    if (r < rows) *reinterpret_cast<uint2*>(q + r * cols + c0 + chunk * 8) = divided_codes8<DT>(raw[u], s, rcp, finite, nan_block);
+  }
+}
+
+// Any strides: a workgroup per 128 x 128 tile, two lanes per row of the tile (64 elements each),
+// dividing element by element. WEIGHT: one scale for the tile, else one per row of the tile.
+// A transposed view (stride_row == 1) still reads neighbouring rows with neighbouring lanes.
+template <int DT, bool WEIGHT>
+__global__ __launch_bounds__(256) void quant_fp8_blocks_generic(const uint16_t* __restrict__ x, int64_t sr, int64_t sc, int64_t rows,
+                                                                int64_t cols, uint8_t* __restrict__ q, float* __restrict__ scale) {
+  saturating_conversions();
+  __shared__ uint32_t wave_amax[4];
+  const int64_t r = (int64_t)blockIdx.y * 128 + (threadIdx.x >> 1);
+  const int64_t c0 = (int64_t)blockIdx.x * 128 + (threadIdx.x & 1) * 64;
+  const bool live = r < rows;
+  const uint16_t* src = x + r * sr + c0 * sc;
+  uint32_t m16 = 0;
+  if (live) {
+    for (int c = 0; c < 64; ++c) {
+      const uint32_t a = src[c * sc] & 0x7FFFu;
+      m16 = a > m16 ? a : m16;
+    }
+  }
+  if constexpr (WEIGHT) {
+    m16 = wave_max(m16);
+    if ((threadIdx.x & 63) == 0) wave_amax[threadIdx.x >> 6] = m16;
+    __syncthreads();
+    m16 = max(max(wave_amax[0], wave_amax[1]), max(wave_amax[2], wave_amax[3]));
+  } else {
+    const uint32_t o = (uint32_t)__shfl_xor((int)m16, 1);
+    m16 = o > m16 ? o : m16;
+  }
+  const float s = scale_of_amax16<DT>(m16);
+  if constexpr (WEIGHT) {
+    if (threadIdx.x == 0) scale[(int64_t)blockIdx.y * gridDim.x + blockIdx.x] = s;
+  } else {
+    if (live && (threadIdx.x & 1) == 0) scale[r * gridDim.x + blockIdx.x] = s;
+  }
+  if (!live) return;
+  const bool finite = m16 < inf16<DT>(), nan_block = m16 > inf16<DT>();
+  uint8_t* dst = q + r * cols + c0;
+  for (int c = 0; c < 64; ++c) dst[c] = (uint8_t)divided_code1<DT>(src[c * sc], s, finite, nan_block);
+}
+
 }  // namespace km
 
 using namespace km;
@@ -873,6 +1000,37 @@ extern "C" int km_quant_rows(const void* x, int64_t rows, int64_t cols, int64_t 
                                              (uint32_t)rows, cols, (uint8_t*)q, scale_out));
   }
   return km_check_launch("km_quant_rows");
+}
+
+extern "C" int km_quant_blocks(const void* x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,
+                               int dtype, int role, void* q, float* scale_out, void* stream) {
+  if (dtype != KM_BF16 && dtype != KM_F16) return km_fail(KM_ERR_ARG, "km_quant_blocks: dtype must be bf16 or f16");
+  if (role != KM_ROLE_ACT && role != KM_ROLE_WEIGHT) return km_fail(KM_ERR_ARG, "km_quant_blocks: role must be KM_ROLE_ACT or KM_ROLE_WEIGHT");
+  if (rows < 0 || cols < 0 || cols % 128) return km_fail(KM_ERR_ARG, "km_quant_blocks: cols must be a non-negative multiple of 128");
+  if (rows == 0 || cols == 0) return KM_OK;
+  if (!x || !q || !scale_out) return km_fail(KM_ERR_ARG, "km_quant_blocks: null pointer");
+  const int64_t tiles_x = cols / 128, tiles_y = (rows + 127) / 128;
+  if (tiles_y > 65535 || tiles_x > 0x7FFFFFFFll) return km_fail(KM_ERR_ARG, "km_quant_blocks: tensor too large");
+  hipStream_t st = (hipStream_t)stream;
+  const uint16_t* xp = (const uint16_t*)x;
+  const dim3 tiles((unsigned)tiles_x, (unsigned)tiles_y);
+  const bool vec = stride_col == 1 && stride_row % 8 == 0 && stride_row >= cols && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(q) & 7) == 0;
+  if (vec && role == KM_ROLE_ACT) {
+    const uint64_t ngroups = (uint64_t)rows * (uint64_t)cols / 8;
+    const uint64_t per_block = (uint64_t)kRowsThreads * kRowsUnroll;
+    const uint64_t blocks = (ngroups + per_block - 1) / per_block;
+    if (blocks > 0x7FFFFFFFull) return km_fail(KM_ERR_ARG, "km_quant_blocks: tensor too large");
+    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL(quant_fp8_blocks_act<DT>, dim3((unsigned)blocks), dim3(kRowsThreads), 0, st, xp, stride_row,
+                                             (uint32_t)(cols / 8), ngroups, (uint8_t*)q, scale_out));
+  } else if (vec) {
+    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL(quant_fp8_blocks_weight<DT>, tiles, dim3(256), 0, st, xp, stride_row, rows, cols, (uint8_t*)q, scale_out));
+  } else if (role == KM_ROLE_ACT) {
+    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL((quant_fp8_blocks_generic<DT, false>), tiles, dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, (uint8_t*)q, scale_out));
+  } else {
+    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL((quant_fp8_blocks_generic<DT, true>), tiles, dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, (uint8_t*)q, scale_out));
+  }
+  return km_check_launch("km_quant_blocks");
 }
 
 extern "C" int km_quant_rows_i8(const void* x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,

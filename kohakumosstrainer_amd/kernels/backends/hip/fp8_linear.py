@@ -6,9 +6,10 @@ quantizer. Host-side counterpart of reference `backends/triton/fp8/linear.py` (c
 
 Recipes served on the GPU: `mx` (block-scaled MFMA; the activation quantizer writes the
 MFMA-packed scales directly, the weight's packed copy comes in `aux` or is packed per call),
-`tensor` (plain fp8 MFMA, scalar scales on the accumulator) and `row` (the same GEMM with one
-scale per output row and one per output column on the accumulator). `block` is not built yet
-and is refused by the support check. The 16-bit input gradient of a base stored
+`tensor` (plain fp8 MFMA, scalar scales on the accumulator), `row` (the same GEMM with one
+scale per output row and one per output column on the accumulator) and `block` (per K block of
+128 the MFMA's partial sum is scaled by the row's and the 128 x 128 weight block's fp32 scales
+and added to the running sum on the vector ALU). The 16-bit input gradient of a base stored
 without a dgrad copy is `dy @ dequantize(W)`: an elementwise dequantize and a plain library
 GEMM, as in the reference's `w16` path.
 """
@@ -24,7 +25,7 @@ from kohakumosstrainer_amd.kernels.fp8.op import make_fp8_linear, make_fp8_linea
 from kohakumosstrainer_amd.kernels.fp8.train import make_fp8_linear_train
 from kohakumosstrainer_amd.kernels.tuning import pow2
 
-GPU_RECIPES = ("mx", "tensor", "row")
+GPU_RECIPES = ("mx", "tensor", "row", "block")
 ALIGN_K = 128
 _RESOLVED: dict[tuple, dict] = {}
 tuning.on_reset(_RESOLVED.clear)
@@ -34,7 +35,8 @@ def candidates(recipe: str, m: int) -> list[dict]:
     """Tile configurations of the fp8 GEMM for M rows, the planner's first pick first: large
     tiles for large M (fewest bytes fetched per flop), smaller ones when M is short or the
     grid would not fill 256 CUs."""
-    cfgs = [{"gemm": "hip", **c} for c in native.configs(native.KERNEL_GEMM_MX if recipe == "mx" else native.KERNEL_GEMM_FP8)]
+    kernel = {"mx": native.KERNEL_GEMM_MX, "block": native.KERNEL_GEMM_BLOCKS}.get(recipe, native.KERNEL_GEMM_FP8)
+    cfgs = [{"gemm": "hip", **c} for c in native.configs(kernel)]
     limit = max(pow2(m, 16), min(c["bm"] for c in cfgs))
     fits = [c for c in cfgs if c["bm"] <= limit] or cfgs
     return sorted(fits, key=lambda c: -(c["bm"] * c["bn"]) if m >= 1024 else c["bm"])
@@ -58,6 +60,9 @@ def _run(cfg, recipe, a, bq, bs, baux, bias):
         if baux is None or baux.numel() != packed_numel(bq.shape[0], bq.shape[1]) or baux.dtype != torch.uint8:
             baux = native.pack_scales(bs)
         return native.gemm_mx(aq, a_packed, bq, baux, bias, a.dtype, cfg["id"], packed=True)
+    if recipe == "block":
+        aq, sa = native.quant_blocks(a, "act")
+        return native.gemm_fp8_blocks(aq, sa, bq, bs.float(), bias, a.dtype, cfg["id"])
     if recipe == "row":
         aq, sa = native.quant_rows(a)
         return native.gemm_fp8_rows(aq, sa, bq, bs.float(), bias, a.dtype, cfg["id"])

@@ -87,10 +87,12 @@ def quantize(x: Tensor, recipe: str, role: str = "act") -> tuple[Tensor, Tensor]
     """`(q e4m3 [rows, K], scale)` of a 2-D operand under `recipe`; `role` matters only for
     `block` (weights scale 128x128 blocks)."""
     _check(x, recipe, role)
-    if x.device.type == "cuda" and x.dtype in _HIP_DTYPES and recipe in ("mx", "tensor", "row") and x.numel():
+    if x.device.type == "cuda" and x.dtype in _HIP_DTYPES and x.numel():
         from kohakumosstrainer_amd import native
 
         x = x.detach()
+        if recipe == "block":
+            return native.quant_blocks(x, role)
         return {"mx": native.quant_mx, "tensor": native.quant_tensor, "row": native.quant_rows}[recipe](x)
     return _quantize_torch(x, recipe, role)
 

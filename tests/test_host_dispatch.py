@@ -98,12 +98,13 @@ def test_supports_and_available_reasons():
     with forced_arch(GFX950):
         assert registry.available("fp8_linear", "cpu", torch.bfloat16, recipe="mx")["hip"] is None
         assert registry.available("fp8_linear", "cpu", torch.bfloat16, recipe="row")["hip"] is None
-        assert "not built" in registry.available("fp8_linear", "cpu", torch.bfloat16, recipe="block")["hip"]
+        assert registry.available("fp8_linear", "cpu", torch.bfloat16, recipe="block")["hip"] is None
+        assert "not built" in registry.available("fp8_linear", "cpu", torch.bfloat16, recipe="nvfp4")["hip"]
         assert registry.available("fp8_linear", "cpu", torch.float32, recipe="mx")["hip"] is not None
         assert registry.available("quant_linear", "cpu", torch.float16, fmt="fp8")["hip"] is None
         assert "unknown" in registry.available("quant_linear", "cpu", torch.float16, fmt="int4")["hip"]
         with pytest.raises(registry.NoImplementationError):
-            registry.resolve("fp8_linear", "cpu", torch.bfloat16, recipe="block")
+            registry.resolve("fp8_linear", "cpu", torch.bfloat16, recipe="nvfp4")
     gate = requires(kinds=("hip",), archs=("gfx950",))
     assert gate(registry.OpQuery("x", CPU, torch.bfloat16)) is not None
     assert gate(registry.OpQuery("x", GFX950, torch.bfloat16)) is None
