@@ -169,24 +169,30 @@ def other_configs(dev, reps):
     }
     # the block recipe (fp32 scales per row x 128 columns / per 128 x 128 weight block), same shape
     wbq, wbs = native.quant_blocks(w, "weight")
-    xbq, xbs = native.quant_blocks(x, "act")
-    bsbuf = torch.empty(m, k // 128, dtype=torch.float32, device=dev)
+    xbq, _, xbs = native.quant_blocks(x, "act", natural=False, kmajor=True)  # the GEMM reads the [K/128, M] scale copy
+    bsbuf = torch.empty(k // 128, m, dtype=torch.float32, device=dev)
 
     def quant_blocks_only():
-        lib.km_quant_blocks(x.data_ptr(), m, k, k, 1, native.KM_BF16, native.ROLE_ACT, qbuf.data_ptr(), bsbuf.data_ptr(), stream)
-
-    def block_step():
-        aq, sa = native.quant_blocks(x, "act")
-        return native.gemm_fp8_blocks(aq, sa, wbq, wbs, bias, torch.bfloat16, 0)
+        lib.km_quant_blocks(x.data_ptr(), m, k, k, 1, native.KM_BF16, native.ROLE_ACT, qbuf.data_ptr(), None, bsbuf.data_ptr(), stream)
 
     quant_blocks_only()
-    block_step()
     qt = event_ms(quant_blocks_only, reps)
-    gt = event_ms(lambda: native.gemm_fp8_blocks(xbq, xbs, wbq, wbs, bias, torch.bfloat16, 0), reps)
+    times = {}
+    for cfg in range(len(native.configs(native.KERNEL_GEMM_BLOCKS))):
+        native.gemm_fp8_blocks(xbq, xbs, wbq, wbs, bias, torch.bfloat16, cfg, kmajor=True)
+        times[cfg] = event_ms(lambda: native.gemm_fp8_blocks(xbq, xbs, wbq, wbs, bias, torch.bfloat16, cfg, kmajor=True), reps)
+    bcfg, gt = min(times.items(), key=lambda kv: kv[1])
+
+    def block_step():
+        aq, _, sa = native.quant_blocks(x, "act", natural=False, kmajor=True)
+        return native.gemm_fp8_blocks(aq, sa, wbq, wbs, bias, torch.bfloat16, bcfg, kmajor=True)
+
+    block_step()
     st = event_ms(block_step, reps)
     out["block_recipe_M16384_K3072_N9216"] = {
         "quant_blocks_us": qt * 1e3, "quant_blocks_GBps": (m * k * 3 + m * (k // 128) * 4) / qt / 1e6, "hbm_peak_GBps": HBM_PEAK_GBS,
-        "gemm_ms": gt, "gemm_TFLOPs": flop / gt / 1e9, "step_ms": st, "step_TFLOPs": flop / st / 1e9, "peak_TFLOPs": FP8_PEAK_TFLOPS,
+        "gemm_ms": gt, "gemm_TFLOPs": flop / gt / 1e9, "gemm_config": bcfg, "gemm_configs_ms": {str(c): t for c, t in times.items()},
+        "step_ms": st, "step_TFLOPs": flop / st / 1e9, "peak_TFLOPs": FP8_PEAK_TFLOPS,
     }
     # int8 compute linear (per-row int8 activations, int8 MFMA GEMM, int32 accumulation), same shape
     w_scale = (w.float().abs().amax(1).clamp_min(1e-12) / 127.0)

@@ -24,7 +24,7 @@ extern "C" {
 enum { KM_OK = 0, KM_ERR_ARG = -1, KM_ERR_LAUNCH = -2, KM_ERR_UNSUPPORTED = -3 };
 enum { KM_BF16 = 0, KM_F16 = 1, KM_F32 = 2 };          /* 16-bit activation / output dtypes */
 enum { KM_Q_INT8 = 0, KM_Q_E4M3 = 1 };                  /* weight-only code formats */
-enum { KM_SCALES_ROWMAJOR = 0, KM_SCALES_PACKED = 1 };  /* MX scale layouts the GEMM reads */
+enum { KM_SCALES_ROWMAJOR = 0, KM_SCALES_PACKED = 1, KM_SCALES_KMAJOR = 2 };  /* scale layouts the GEMMs read */
 enum { KM_KERNEL_GEMM_MX = 0, KM_KERNEL_GEMM_FP8 = 1, KM_KERNEL_WO_FWD = 2, KM_KERNEL_WO_DGRAD = 3, KM_KERNEL_GEMM_BLOCKS = 4 };
 enum { KM_ROLE_ACT = 0, KM_ROLE_WEIGHT = 1 };                     /* operand roles of the block recipe */
 
@@ -73,14 +73,16 @@ int km_quant_rows(const void *x, int64_t rows, int64_t cols, int64_t stride_row,
                   int dtype, void *q, float *scale_out, void *stream);
 
 /* Block-recipe e4m3 quantizer (cols % 128 == 0, any strides). KM_ROLE_ACT: one scale per row and
- * 128 columns, scale_out [rows, cols/128]; KM_ROLE_WEIGHT: one scale per 128 x 128 block (rows past
- * the end count as zeros), scale_out [ceil(rows/128), cols/128]. scale = max(amax, 1e-12) / 448 and
+ * 128 columns, scale_out [rows, cols/128] (the reference's layout) and / or scale_kmajor
+ * [cols/128, rows], the copy km_gemm_fp8_blocks reads fastest (either may be NULL, not both);
+ * KM_ROLE_WEIGHT: one scale per 128 x 128 block (rows past the end count as zeros), scale_out
+ * [ceil(rows/128), cols/128], scale_kmajor NULL. scale = max(amax, 1e-12) / 448 and
  * q = e4m3(clamp(x / scale)), both IEEE divisions. q is [rows, cols] contiguous.
  * Replaces fp8.formats.quantize(x, "block", role) (src/kohakumoss_kernels/fp8/formats.py:83-93)
  * and, for activations, Triton quantize_blocks(x, mx=False) (backends/triton/fp8/quantize.py:95-119,
  * 171-187); the reference quantizes weight blocks with the eager formats only. */
 int km_quant_blocks(const void *x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,
-                    int dtype, int role, void *q, float *scale_out, void *stream);
+                    int dtype, int role, void *q, float *scale_out, float *scale_kmajor, void *stream);
 
 /* Per-row int8 quantizer of the int8 compute linear: v = x (* col_scale[c], in fp32, when col_scale
  * is not NULL; [cols] fp32), scale_out[r] = max(amax of row r of v, 1e-12) / 127 (IEEE division),
@@ -118,13 +120,14 @@ int km_gemm_fp8_rows(const void *a, const float *sa, const void *b, const float 
                      int config, void *stream);
 
 /* Block-recipe fp8 GEMM: C[m,n] = sum over K blocks kb of (A[m,kb] . B[n,kb]) * sa[m,kb] * sb[n/128,kb]
- * + bias[n]; sa [M, K/128] and sb [ceil(N/128), K/128] fp32, contiguous. Each block's partial product
- * is accumulated in fp32 on the MFMA and promoted (scaled and added to the running fp32 sum) on the
- * vector ALU. K % 128 == 0; config < km_num_configs(KM_KERNEL_GEMM_BLOCKS).
+ * + bias[n]; sb [ceil(N/128), K/128] fp32; sa fp32 in the layout sa_layout names: KM_SCALES_ROWMAJOR
+ * [M, K/128] or KM_SCALES_KMAJOR [K/128, M] (faster: the 16 rows of an MFMA tile read one run).
+ * Each block's partial product is accumulated in fp32 on the MFMA and promoted (scaled and added
+ * to the running fp32 sum) on the vector ALU. K % 128 == 0; config < km_num_configs(KM_KERNEL_GEMM_BLOCKS).
  * Replaces Triton promote_mm with sub = 128, b_rows = 128 (backends/triton/fp8/gemm.py:108-134,205-216). */
 int km_gemm_fp8_blocks(const void *a, const float *sa, const void *b, const float *sb,
                        const void *bias, void *c, int64_t M, int64_t N, int64_t K, int out_dtype,
-                       int config, void *stream);
+                       int sa_layout, int config, void *stream);
 
 /* int8 GEMM with int32 accumulation: C[m,n] = ((float(A B^T)[m,n] * sa[m]) * sb[n]) + bias[n], every
  * product and the sum rounded to fp32 on its own and the result once to out_dtype, which makes

@@ -31,8 +31,13 @@ def hipcc() -> str:
     return path
 
 
+# Per-file additions. The block-recipe GEMM promotes MFMA results on the vector ALU: the MFMAs must
+# write ordinary vector registers, or every partial sum is first copied out of an accumulation register.
+EXTRA_FLAGS = {"km_gemm_blocks.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def _compile(src: Path, obj: Path) -> None:
-    cmd = [hipcc(), f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-c", str(src), "-o", str(obj), *DEVICE_FLAGS]
+    cmd = [hipcc(), f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-c", str(src), "-o", str(obj), *DEVICE_FLAGS, *EXTRA_FLAGS.get(src.name, [])]
     done = subprocess.run(cmd, capture_output=True, text=True)
     if done.returncode:
         raise RuntimeError(f"hipcc failed on {src.name}:\n{done.stderr[-6000:]}")

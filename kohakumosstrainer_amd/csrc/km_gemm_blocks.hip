@@ -10,33 +10,45 @@
 // Replaces the reference's Triton _promote_kernel with SUB = 128, B_ROWS = 128
 // (src/kohakumoss_kernels/backends/triton/fp8/gemm.py:108-134,205-216).
 //
-// Shape of the kernel. A workgroup of four wavefronts (2 x 2) owns a 128 x 128 tile, so the
-// weight scale is one number per workgroup and K step; a wavefront's 64 x 64 sub-tile is 16 MFMA
-// tiles: 64 registers of partial sums and 64 of running sums per lane, which leaves room for two
-// workgroups per compute unit (one's vector-ALU promotion runs under the other's MFMAs). The
-// operand slabs of step k+1 are requested (direct-to-LDS buffer loads, double buffered, the
-// swizzled slab layout of the other fp8 GEMMs) before the MFMAs of step k are issued and waited
-// for after them.
+// Shape of the kernel. A workgroup of four wavefronts (2 x 2) owns a BM x 128 tile, so the weight
+// scale is one number per workgroup and K step. A wavefront's (BM/2) x 64 sub-tile is walked in
+// rows of four MFMA tiles (16 tokens x 64 output columns, which share one activation scale): the
+// four MFMAs of a row write a set of partial-sum registers, and between them the partial sums of
+// the row before (the other set) are promoted on the vector ALU, so the promotion is issued while
+// the matrix pipe is busy. The B fragments of a step stay in registers; A fragments are read a row
+// ahead. The operand slabs are fetched STAGES - 1 steps ahead (direct-to-LDS buffer loads into a
+// ring of STAGES buffers, the swizzled slab layout of the other fp8 GEMMs); a step waits only for
+// the slabs of the step after it, so the fetches of the step after that stay in flight across the
+// barrier. The tall tile halves the LDS reads per MFMA of the square one (LDS bandwidth, not the
+// matrix pipe, bounds 64 x 64 sub-tiles).
 #include <stdio.h>
 
 #include "km_gemm_common.h"
 
 namespace km {
 
-constexpr int kBlkTile = 128;
+constexpr int kBlkTileN = 128;
 
-template <int OUT>
-__global__ __launch_bounds__(256, 2) void gemm_fp8_blocks_kernel(
+// Built with -mllvm -amdgpu-mfma-vgpr-form: the MFMAs write ordinary vector registers. Without it
+// the compiler puts their results in accumulation registers and copies every partial sum out
+// before the promotion (one more vector-ALU instruction per value).
+// SA_KMAJOR: the activation scales are laid out [K/128, M] (the quantizer's second output), so
+// the 16 rows of an MFMA tile read one 64-byte run per step; from the natural [M, K/128] matrix
+// every lane gathers from a row of its own, which costs more than the MFMAs of the step.
+template <int OUT, int BM, int STAGES, bool SA_KMAJOR>
+__global__ __launch_bounds__(256) void gemm_fp8_blocks_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const float* __restrict__ sa,
     const float* __restrict__ sb, const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N, int K) {
-  constexpr int BM = kBlkTile, BN = kBlkTile;
-  constexpr int TM = BM / 32, TN = BN / 32;  // 16x16 MFMA tiles per wavefront and axis
-  constexpr int SLAB = BM * kStepBytes;      // 16 KiB
-  constexpr int PASSES = BM / 32;            // 4 KiB (32 rows) per pass of 256 lanes
-  __shared__ __attribute__((aligned(1024))) uint8_t a_buf0[SLAB];
-  __shared__ __attribute__((aligned(1024))) uint8_t a_buf1[SLAB];
-  __shared__ __attribute__((aligned(1024))) uint8_t b_buf0[SLAB];
-  __shared__ __attribute__((aligned(1024))) uint8_t b_buf1[SLAB];
+  constexpr int BN = kBlkTileN;
+  constexpr int TM = BM / 32, TN = BN / 32;     // 16x16 MFMA tiles per wavefront and axis
+  constexpr int A_SLAB = BM * kStepBytes, B_SLAB = BN * kStepBytes;
+  constexpr int A_PASSES = BM / 32, B_PASSES = BN / 32;  // 32 rows (4 KiB) per pass of 256 lanes
+  constexpr int DMAS = A_PASSES + B_PASSES;     // slab fetch instructions per wavefront and step
+  static_assert(STAGES == 2 || STAGES == 3, "ring of two or three slab pairs");
+  static_assert(STAGES * (A_SLAB + B_SLAB) <= 160 * 1024, "LDS");
+  static_assert(STAGES * A_SLAB >= 2 * 16384 && STAGES * B_SLAB >= 2 * 16384, "epilogue staging: four 16 KiB buffers");
+  __shared__ __attribute__((aligned(1024))) uint8_t a_ring[STAGES][A_SLAB];
+  __shared__ __attribute__((aligned(1024))) uint8_t b_ring[STAGES][B_SLAB];
 
   int tile_m, tile_n;
   tile_of(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, tile_n);
@@ -59,9 +71,9 @@ __global__ __launch_bounds__(256, 2) void gemm_fp8_blocks_kernel(
   auto dma = [&](uint8_t* abuf, uint8_t* bbuf, int ks) __attribute__((always_inline)) {
     const int koff = __builtin_amdgcn_readfirstlane(ks * kStepBytes);
 #pragma unroll
-    for (int i = 0; i < PASSES; ++i) hidden_dma_b128(a_rsrc, lds_offset(abuf) + i * 4096 + wave * 1024, ld_voff + i * pass_stride, koff);
+    for (int i = 0; i < A_PASSES; ++i) hidden_dma_b128(a_rsrc, lds_offset(abuf) + i * 4096 + wave * 1024, ld_voff + i * pass_stride, koff);
 #pragma unroll
-    for (int i = 0; i < PASSES; ++i) hidden_dma_b128(b_rsrc, lds_offset(bbuf) + i * 4096 + wave * 1024, ld_voff + i * pass_stride, koff);
+    for (int i = 0; i < B_PASSES; ++i) hidden_dma_b128(b_rsrc, lds_offset(bbuf) + i * 4096 + wave * 1024, ld_voff + i * pass_stride, koff);
   };
   auto fragment = [&](const uint8_t* slab, int row) __attribute__((always_inline)) -> v8i {
     const v4i lo = *reinterpret_cast<const v4i*>(slab + slab_offset(row, g));
@@ -69,11 +81,30 @@ __global__ __launch_bounds__(256, 2) void gemm_fp8_blocks_kernel(
     return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
 
-  // scales of this lane's TM token rows (clamped to the last row) and of the tile's weight block
-  const float* sa_row[TM];
-#pragma unroll
-  for (int j = 0; j < TM; ++j) sa_row[j] = sa + (size_t)min(m0 + wm + j * 16 + r16, M - 1) * nk;
+  // Scales of this lane's TM token rows and of the tile's weight block.
+  // The activation scales are fetched like the slabs, from inline asm: a load the compiler sees
+  // would make it wait for every fetch in flight (its count does not include the hidden ones)
+  // where the value is first used. The fetched registers are read once, by an opaque move placed
+  // right after the step's own wait.
+  // The descriptor starts at this tile's first row: rows past M read as zero scales (their
+  // partial sums are zeros as well). Row j * 16 + r16 of the sub-tile: the lane part of the
+  // offset is one register, the row-group part is uniform.
+  // (K-major: a row past M reads a neighbour's scale or, past the end, zero; its sums are never stored.)
+  const v4i sa_rsrc = SA_KMAJOR ? raw_rsrc(sa, (uint32_t)min((int64_t)M * nk * 4, (int64_t)0x7FFFFFFF))
+                                : raw_rsrc(sa + (size_t)m0 * nk, (uint32_t)min((int64_t)(M - m0) * nk * 4, (int64_t)0x7FFFFFFF));
+  const int sa_voff = SA_KMAJOR ? (m0 + wm + r16) * 4 : (wm + r16) * nk * 4;
   const float* sb_row = sb + (size_t)tile_n * nk;
+  uint32_t sa_raw[TM];
+  auto sa_fetch = [&](int ks) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+      sa_raw[j] = hidden_load_b32(sa_rsrc, sa_voff, __builtin_amdgcn_readfirstlane(SA_KMAJOR ? (ks * M + j * 16) * 4 : (ks + j * 16 * nk) * 4));
+  };
+  float sa_next[TM];
+  auto sa_take = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < TM; ++j) asm volatile("v_mov_b32 %0, %1" : "=v"(sa_next[j]) : "v"(sa_raw[j]));
+  };
 
   v4f acc[TN][TM];
 #pragma unroll
@@ -81,74 +112,114 @@ __global__ __launch_bounds__(256, 2) void gemm_fp8_blocks_kernel(
 #pragma unroll
     for (int j = 0; j < TM; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
-  // raw scales of the step ahead: loaded a step early, multiplied once that step begins
-  float sa_next[TM], sb_next = sb_row[0];
-#pragma unroll
-  for (int j = 0; j < TM; ++j) sa_next[j] = sa_row[j][0];
-  dma(a_buf0, b_buf0, 0);
-  __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+  // raw scales of the step ahead: fetched a step early, multiplied once that step begins
+  float sb_next = sb_row[0];
+  // prologue: the scales of step 0 and the slabs of the first STAGES - 1 steps; wait for step 0 only
+  sa_fetch(0);
+  dma(a_ring[0], b_ring[0], 0);
+  if (STAGES == 3 && nk > 1) {
+    dma(a_ring[1], b_ring[1], 1);
+    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(DMAS));
+  } else {
+    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+  }
   __syncthreads();
+  __builtin_amdgcn_sched_barrier(0);
+  sa_take();
 
-  auto step = [&](const uint8_t* a_cur, const uint8_t* b_cur, uint8_t* a_nxt, uint8_t* b_nxt, int ks) __attribute__((always_inline)) {
+  // One K step: the slabs of step ks are in ring slot `cur`; slot `pre` (read last in the step
+  // before, behind that step's barrier) takes the slabs of step ks + STAGES - 1.
+  auto step = [&](int ks, auto cur_tag, auto pre_tag) __attribute__((always_inline)) {
+    constexpr int cur = decltype(cur_tag)::value, pre = decltype(pre_tag)::value;
+    const uint8_t* a_cur = a_ring[cur];
+    const uint8_t* b_cur = b_ring[cur];
     float s_cur[TM];
 #pragma unroll
     for (int j = 0; j < TM; ++j) s_cur[j] = sa_next[j] * sb_next;
-    if (ks + 1 < nk) {
-      // the other pair of buffers was last read in the step before, behind that step's barrier
-      sb_next = sb_row[ks + 1];
+    sb_next = sb_row[min(ks + 1, nk - 1)];
+    sa_fetch(min(ks + 1, nk - 1));
+    const bool ahead = ks + STAGES - 1 < nk;
+    if (ahead) dma(a_ring[pre], b_ring[pre], ks + STAGES - 1);
+    v8i wf[TN];
 #pragma unroll
-      for (int j = 0; j < TM; ++j) sa_next[j] = sa_row[j][ks + 1];
-      dma(a_nxt, b_nxt, ks + 1);
-    }
-    v8i xf[TM];
+    for (int t = 0; t < TN; ++t) wf[t] = fragment(b_cur, wn + t * 16 + r16);
+    v8i xf = fragment(a_cur, wm + r16);
+    v4f part[2][TN];
+    static_for<TM + 1>([&](auto j_tag) __attribute__((always_inline)) {
+      constexpr int j = decltype(j_tag)::value;
+      v8i xf_next = xf;
+      if constexpr (j + 1 < TM) xf_next = fragment(a_cur, wm + (j + 1) * 16 + r16);
+      static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
+        constexpr int t = decltype(t_tag)::value;
+        // MFMA rows come from B (output columns n), MFMA columns from A (tokens m); unit scales
+        if constexpr (j < TM)
+          part[j & 1][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[t], xf, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+        if constexpr (j > 0) {
 #pragma unroll
-    for (int j = 0; j < TM; ++j) xf[j] = fragment(a_cur, wm + j * 16 + r16);
-    v8i wf = fragment(b_cur, wn + r16);
-    // The four MFMAs of a row of tiles are issued back to back; the sums of the row before are
-    // promoted on the vector ALU while they run (two sets of partial-sum registers).
-    v4f part[2][TM];
-    static_for<TN + 1>([&](auto t_tag) __attribute__((always_inline)) {
-      constexpr int t = decltype(t_tag)::value;
-      if constexpr (t < TN) {
-        v8i wf_next = wf;
-        if constexpr (t + 1 < TN) wf_next = fragment(b_cur, wn + (t + 1) * 16 + r16);
-#pragma unroll
-        for (int j = 0; j < TM; ++j) {
-          // MFMA rows come from B (output columns n), MFMA columns from A (tokens m); unit scales
-          part[t & 1][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
-        }
-        wf = wf_next;
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      if constexpr (t > 0) {
-#pragma unroll
-        for (int j = 0; j < TM; ++j) {
-#pragma unroll
-          for (int v = 0; v < 4; ++v) acc[t - 1][j][v] = __builtin_fmaf(part[(t - 1) & 1][j][v], s_cur[j], acc[t - 1][j][v]);
+          for (int v = 0; v < 4; ++v) acc[t][j - 1][v] = __builtin_fmaf(part[(j - 1) & 1][t][v], s_cur[j - 1], acc[t][j - 1][v]);
           // pins the promotion ahead of the wait below (the compiler would sink it past the barrier)
-          asm volatile("" : "+v"(acc[t - 1][j]));
+          asm volatile("" : "+v"(acc[t][j - 1]));
         }
-      }
-      __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      xf = xf_next;
     });
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));  // the slabs of the next step have landed, this step's LDS reads are done
+    // The slabs and scales of step ks + 1 must have landed (STAGES 3: the DMAS newest fetches, those
+    // of step ks + 2, stay in flight: vector-memory results return in order) and this step's LDS reads
+    // must be done before the barrier lets another wavefront overwrite the slot.
+    if (STAGES == 3 && ahead) __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(DMAS));
+    else __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
+    sa_take();
   };
-  for (int ks = 0; ks < nk; ks += 2) {
-    step(a_buf0, b_buf0, a_buf1, b_buf1, ks);
-    if (ks + 1 < nk) step(a_buf1, b_buf1, a_buf0, b_buf0, ks + 1);
+  using i0 = std::integral_constant<int, 0>;
+  using i1 = std::integral_constant<int, 1>;
+  using i2 = std::integral_constant<int, 2>;
+  if constexpr (STAGES == 2) {
+    for (int ks = 0; ks < nk; ks += 2) {
+      step(ks, i0{}, i1{});
+      if (ks + 1 < nk) step(ks + 1, i1{}, i0{});
+    }
+  } else {
+    for (int ks = 0; ks < nk; ks += 3) {
+      step(ks, i0{}, i2{});
+      if (ks + 1 < nk) step(ks + 1, i1{}, i0{});
+      if (ks + 2 < nk) step(ks + 2, i2{}, i1{});
+    }
   }
 
-  store_tile<BM, BN, OUT, 0>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, m0, n0, a_buf0, a_buf1, b_buf0, b_buf1);
+  // every fetch has landed and every wavefront is past its last LDS read: the ring is free
+  uint8_t* ea = &a_ring[0][0];
+  uint8_t* eb = &b_ring[0][0];
+  store_tile<BM, BN, OUT, 0, false>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, m0, n0, ea, ea + 16384, eb, eb + 16384);
 }
 
-int blocks_gemm_num_configs() { return 1; }
+struct BlocksConfig {
+  int bm, stages;
+};
+// the tall tile first (fewest operand and LDS bytes per flop); the square one for short M and small grids
+static const BlocksConfig kBlocksConfigs[] = {{256, 3}, {128, 2}};
+constexpr int kNumBlocksConfigs = 2;
+
+int blocks_gemm_num_configs() { return kNumBlocksConfigs; }
 int blocks_gemm_config_desc(int config, char* buf, int len) {
-  if (config != 0) return km_fail(KM_ERR_ARG, "config out of range");
-  snprintf(buf, len, "bm=%d,bn=%d,bk=128,waves=4,wg_per_cu=2", kBlkTile, kBlkTile);
+  if (config < 0 || config >= kNumBlocksConfigs) return km_fail(KM_ERR_ARG, "config out of range");
+  const BlocksConfig& c = kBlocksConfigs[config];
+  snprintf(buf, len, "bm=%d,bn=%d,bk=128,waves=4,stages=%d,wg_per_cu=%d", c.bm, kBlkTileN, c.stages, c.bm == 256 ? 1 : 2);
   return KM_OK;
+}
+
+template <int OUT, int BM, int STAGES>
+static void launch_blocks(const void* a, const float* sa, const void* b, const float* sb, const void* bias, void* c,
+                          int M, int N, int K, bool sa_kmajor, hipStream_t st) {
+  const int tiles = ((M + BM - 1) / BM) * ((N + kBlkTileN - 1) / kBlkTileN);
+  if (sa_kmajor)
+    hipLaunchKernelGGL((gemm_fp8_blocks_kernel<OUT, BM, STAGES, true>), dim3(tiles), dim3(256), 0, st, (const uint8_t*)a,
+                       (const uint8_t*)b, sa, sb, (const uint16_t*)bias, (uint16_t*)c, M, N, K);
+  else
+    hipLaunchKernelGGL((gemm_fp8_blocks_kernel<OUT, BM, STAGES, false>), dim3(tiles), dim3(256), 0, st, (const uint8_t*)a,
+                       (const uint8_t*)b, sa, sb, (const uint16_t*)bias, (uint16_t*)c, M, N, K);
 }
 
 }  // namespace km
@@ -157,23 +228,25 @@ using namespace km;
 
 extern "C" int km_gemm_fp8_blocks(const void* a, const float* sa, const void* b, const float* sb,
                                   const void* bias, void* c, int64_t M, int64_t N, int64_t K,
-                                  int out_dtype, int config, void* stream) {
+                                  int out_dtype, int sa_layout, int config, void* stream) {
   if (out_dtype != KM_BF16 && out_dtype != KM_F16) return km_fail(KM_ERR_ARG, "km_gemm_fp8_blocks: out_dtype must be bf16 or f16");
   if (M < 0 || N < 0 || K <= 0 || K % kStepBytes) return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_fp8_blocks: K must be a positive multiple of 128");
   if (M * K > 0x7FFFFFFFll || N * K > 0x7FFFFFFFll || M > 0x0FFFFFFF || N > 0x0FFFFFFF)
     return km_fail(KM_ERR_ARG, "km_gemm_fp8_blocks: dimension too large");
-  if (config != 0) return km_fail(KM_ERR_ARG, "km_gemm_fp8_blocks: config out of range");
+  if (config < 0 || config >= kNumBlocksConfigs) return km_fail(KM_ERR_ARG, "km_gemm_fp8_blocks: config out of range");
+  if (sa_layout != KM_SCALES_ROWMAJOR && sa_layout != KM_SCALES_KMAJOR) return km_fail(KM_ERR_ARG, "km_gemm_fp8_blocks: unknown activation scale layout");
   if (M == 0 || N == 0) return KM_OK;
   if (!a || !b || !c || !sa || !sb) return km_fail(KM_ERR_ARG, "km_gemm_fp8_blocks: null pointer");
   if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15)
     return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_fp8_blocks: operands must be 16-byte aligned");
-  const int tiles = (int)(((M + kBlkTile - 1) / kBlkTile) * ((N + kBlkTile - 1) / kBlkTile));
   hipStream_t st = (hipStream_t)stream;
-  if (out_dtype == KM_BF16)
-    hipLaunchKernelGGL(gemm_fp8_blocks_kernel<KM_BF16>, dim3(tiles), dim3(256), 0, st, (const uint8_t*)a, (const uint8_t*)b, sa, sb,
-                       (const uint16_t*)bias, (uint16_t*)c, (int)M, (int)N, (int)K);
-  else
-    hipLaunchKernelGGL(gemm_fp8_blocks_kernel<KM_F16>, dim3(tiles), dim3(256), 0, st, (const uint8_t*)a, (const uint8_t*)b, sa, sb,
-                       (const uint16_t*)bias, (uint16_t*)c, (int)M, (int)N, (int)K);
+  const bool km = sa_layout == KM_SCALES_KMAJOR;
+  if (out_dtype == KM_BF16) {
+    if (config == 0) launch_blocks<KM_BF16, 256, 3>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
+    else launch_blocks<KM_BF16, 128, 2>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
+  } else {
+    if (config == 0) launch_blocks<KM_F16, 256, 3>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
+    else launch_blocks<KM_F16, 128, 2>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
+  }
   return km_check_launch("km_gemm_fp8_blocks");
 }

@@ -124,13 +124,16 @@ __device__ __forceinline__ uint32_t hidden_load_b32(const v4i& rsrc, int voffset
 // SCALED 0: acc + bias; 1: acc * (row * col scale) + bias, fused; 2: the accumulator holds int32
 // bits: ((float(acc) * row scale) * col scale) + bias with every product and the sum rounded
 // on its own, the order of the reference's int8 linear (src/kohakumoss_kernels/int8/op.py:45-48).
-template <int BM, int BN, int OUT, int SCALED>
+// A workgroup of eight wavefronts calls it once per group of four (wavefront index modulo 4,
+// m0 of that group's rows) with SYNC off, after a barrier of its own: the groups may take
+// different branches here.
+template <int BM, int BN, int OUT, int SCALED, bool SYNC = true>
 __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float post, const float* __restrict__ row_scale,
                                            const float* __restrict__ col_scale, const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N,
                                            int m0, int n0, uint8_t* buf0, uint8_t* buf1, uint8_t* buf2, uint8_t* buf3) {
   constexpr int WTM = BM / 2, WTN = BN / 2, TM = WTM / 16, TN = WTN / 16;
   const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) & 3;
   const int wm = (wave >> 1) * WTM, wn = (wave & 1) * WTN;
   const int r16 = lane & 15, g = lane >> 4;
   const bool has_bias = bias != nullptr;
@@ -156,7 +159,7 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
     constexpr int LPR = WTN * 2 / 16;           // lanes per row on the read side
     constexpr int RPI = 64 / LPR;               // rows per read instruction
     static_assert(HM * 16 * RP <= kMinBuf, "epilogue staging: one buffer per wavefront");
-    __syncthreads();  // every wavefront is done reading fragments
+    if constexpr (SYNC) __syncthreads();  // every wavefront is done reading fragments
     uint8_t* region = wave == 0 ? buf0 : wave == 1 ? buf1 : wave == 2 ? buf2 : buf3;
     const uint16_t* bias_lane = bias + (has_bias ? n0 + wn + 4 * g : 0);
     float bv[TN][4], cs[TN][4];

@@ -759,7 +759,8 @@ __device__ __forceinline__ uint32_t row16_max(uint32_t v) {
 // q and the scales [rows, cols/128] are contiguous, so both are indexed by the flat group number.
 template <int DT>
 __global__ __launch_bounds__(kRowsThreads) void quant_fp8_blocks_act(const uint16_t* __restrict__ x, int64_t ld, uint32_t groups_per_row,
-                                                                     uint64_t ngroups, uint8_t* __restrict__ q, float* __restrict__ scale) {
+                                                                     uint64_t ngroups, uint32_t rows, uint8_t* __restrict__ q, float* __restrict__ scale,
+                                                                     float* __restrict__ scale_km) {
   saturating_conversions();
   const uint64_t base = (uint64_t)blockIdx.x * (kRowsThreads * kRowsUnroll) + threadIdx.x;
   const bool dense = ld == (int64_t)groups_per_row * 8;
@@ -788,7 +789,14 @@ __global__ __launch_bounds__(kRowsThreads) void quant_fp8_blocks_act(const uint1
     const uint2 codes = divided_codes8<DT>(raw[u], s, rcp, m16 < inf16<DT>(), m16 > inf16<DT>());
     if (g < ngroups) {
       *reinterpret_cast<uint2*>(q + g * 8) = codes;
-      if ((threadIdx.x & 15) == 0) scale[g >> 4] = s;
+      if ((threadIdx.x & 15) == 0) {
+        if (scale) scale[g >> 4] = s;
+        if (scale_km) {  // [cols/128, rows]: the layout the GEMM reads with one run per 16 rows
+          const uint32_t blocks = groups_per_row >> 4;
+          const uint64_t b = g >> 4, row = b / blocks;
+          scale_km[(b - row * blocks) * rows + row] = s;
+        }
+      }
     }
   }
 }
@@ -830,11 +838,13 @@ __global__ __launch_bounds__(256) void quant_fp8_blocks_weight(const uint16_t* _
 }
 
 // Any strides: a workgroup per 128 x 128 tile, two lanes per row of the tile (64 elements each),
-// dividing element by element. WEIGHT: one scale for the tile, else one per row of the tile.
+// dividing element by element. WEIGHT: one scale for the tile, else one per row of the tile (and
+// its [cols/128, rows] copy when asked for).
 // A transposed view (stride_row == 1) still reads neighbouring rows with neighbouring lanes.
 template <int DT, bool WEIGHT>
 __global__ __launch_bounds__(256) void quant_fp8_blocks_generic(const uint16_t* __restrict__ x, int64_t sr, int64_t sc, int64_t rows,
-                                                                int64_t cols, uint8_t* __restrict__ q, float* __restrict__ scale) {
+                                                                int64_t cols, uint8_t* __restrict__ q, float* __restrict__ scale,
+                                                                float* __restrict__ scale_km) {
   saturating_conversions();
   __shared__ uint32_t wave_amax[4];
   const int64_t r = (int64_t)blockIdx.y * 128 + (threadIdx.x >> 1);
@@ -861,7 +871,10 @@ __global__ __launch_bounds__(256) void quant_fp8_blocks_generic(const uint16_t* 
   if constexpr (WEIGHT) {
     if (threadIdx.x == 0) scale[(int64_t)blockIdx.y * gridDim.x + blockIdx.x] = s;
   } else {
-    if (live && (threadIdx.x & 1) == 0) scale[r * gridDim.x + blockIdx.x] = s;
+    if (live && (threadIdx.x & 1) == 0) {
+      if (scale) scale[r * gridDim.x + blockIdx.x] = s;
+      if (scale_km) scale_km[(int64_t)blockIdx.x * rows + r] = s;
+    }
   }
   if (!live) return;
   const bool finite = m16 < inf16<DT>(), nan_block = m16 > inf16<DT>();
@@ -1003,12 +1016,14 @@ extern "C" int km_quant_rows(const void* x, int64_t rows, int64_t cols, int64_t 
 }
 
 extern "C" int km_quant_blocks(const void* x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,
-                               int dtype, int role, void* q, float* scale_out, void* stream) {
+                               int dtype, int role, void* q, float* scale_out, float* scale_kmajor, void* stream) {
   if (dtype != KM_BF16 && dtype != KM_F16) return km_fail(KM_ERR_ARG, "km_quant_blocks: dtype must be bf16 or f16");
   if (role != KM_ROLE_ACT && role != KM_ROLE_WEIGHT) return km_fail(KM_ERR_ARG, "km_quant_blocks: role must be KM_ROLE_ACT or KM_ROLE_WEIGHT");
   if (rows < 0 || cols < 0 || cols % 128) return km_fail(KM_ERR_ARG, "km_quant_blocks: cols must be a non-negative multiple of 128");
   if (rows == 0 || cols == 0) return KM_OK;
-  if (!x || !q || !scale_out) return km_fail(KM_ERR_ARG, "km_quant_blocks: null pointer");
+  if (!x || !q || (!scale_out && !scale_kmajor)) return km_fail(KM_ERR_ARG, "km_quant_blocks: null pointer");
+  if (role == KM_ROLE_WEIGHT && (scale_kmajor || !scale_out)) return km_fail(KM_ERR_ARG, "km_quant_blocks: weight blocks have the one scale layout");
+  if (rows > 0x7FFFFFFFll) return km_fail(KM_ERR_ARG, "km_quant_blocks: too many rows");
   const int64_t tiles_x = cols / 128, tiles_y = (rows + 127) / 128;
   if (tiles_y > 65535 || tiles_x > 0x7FFFFFFFll) return km_fail(KM_ERR_ARG, "km_quant_blocks: tensor too large");
   hipStream_t st = (hipStream_t)stream;
@@ -1022,13 +1037,13 @@ extern "C" int km_quant_blocks(const void* x, int64_t rows, int64_t cols, int64_
     const uint64_t blocks = (ngroups + per_block - 1) / per_block;
     if (blocks > 0x7FFFFFFFull) return km_fail(KM_ERR_ARG, "km_quant_blocks: tensor too large");
     KM_DISPATCH_DT(dtype, hipLaunchKernelGGL(quant_fp8_blocks_act<DT>, dim3((unsigned)blocks), dim3(kRowsThreads), 0, st, xp, stride_row,
-                                             (uint32_t)(cols / 8), ngroups, (uint8_t*)q, scale_out));
+                                             (uint32_t)(cols / 8), ngroups, (uint32_t)rows, (uint8_t*)q, scale_out, scale_kmajor));
   } else if (vec) {
     KM_DISPATCH_DT(dtype, hipLaunchKernelGGL(quant_fp8_blocks_weight<DT>, tiles, dim3(256), 0, st, xp, stride_row, rows, cols, (uint8_t*)q, scale_out));
   } else if (role == KM_ROLE_ACT) {
-    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL((quant_fp8_blocks_generic<DT, false>), tiles, dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, (uint8_t*)q, scale_out));
+    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL((quant_fp8_blocks_generic<DT, false>), tiles, dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, (uint8_t*)q, scale_out, scale_kmajor));
   } else {
-    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL((quant_fp8_blocks_generic<DT, true>), tiles, dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, (uint8_t*)q, scale_out));
+    KM_DISPATCH_DT(dtype, hipLaunchKernelGGL((quant_fp8_blocks_generic<DT, true>), tiles, dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, (uint8_t*)q, scale_out, (float*)nullptr));
   }
   return km_check_launch("km_quant_blocks");
 }

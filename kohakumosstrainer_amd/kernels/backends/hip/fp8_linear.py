@@ -61,8 +61,8 @@ def _run(cfg, recipe, a, bq, bs, baux, bias):
             baux = native.pack_scales(bs)
         return native.gemm_mx(aq, a_packed, bq, baux, bias, a.dtype, cfg["id"], packed=True)
     if recipe == "block":
-        aq, sa = native.quant_blocks(a, "act")
-        return native.gemm_fp8_blocks(aq, sa, bq, bs.float(), bias, a.dtype, cfg["id"])
+        aq, _, sa_t = native.quant_blocks(a, "act", natural=False, kmajor=True)
+        return native.gemm_fp8_blocks(aq, sa_t, bq, bs.float(), bias, a.dtype, cfg["id"], kmajor=True)
     if recipe == "row":
         aq, sa = native.quant_rows(a)
         return native.gemm_fp8_rows(aq, sa, bq, bs.float(), bias, a.dtype, cfg["id"])

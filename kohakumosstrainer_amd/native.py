@@ -21,7 +21,7 @@ KM_Q_INT8, KM_Q_E4M3 = 0, 1
 KERNEL_GEMM_MX, KERNEL_GEMM_FP8, KERNEL_WO_FWD, KERNEL_WO_DGRAD, KERNEL_GEMM_BLOCKS = 0, 1, 2, 3, 4
 ROLE_ACT, ROLE_WEIGHT = 0, 1
 BLOCK = 128
-SCALES_ROWMAJOR, SCALES_PACKED = 0, 1
+SCALES_ROWMAJOR, SCALES_PACKED, SCALES_KMAJOR = 0, 1, 2
 _DTYPES = {torch.bfloat16: KM_BF16, torch.float16: KM_F16}
 _QFORMATS = {torch.int8: KM_Q_INT8, E4M3: KM_Q_E4M3}
 
@@ -69,12 +69,12 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.km_scales_pack.argtypes = [p, i64, i64, p, p]
     lib.km_quant_tensor.argtypes = [p, i64, i64, i64, i64, i32, p, p, p, p]
     lib.km_quant_rows.argtypes = [p, i64, i64, i64, i64, i32, p, p, p]
-    lib.km_quant_blocks.argtypes = [p, i64, i64, i64, i64, i32, i32, p, p, p]
+    lib.km_quant_blocks.argtypes = [p, i64, i64, i64, i64, i32, i32, p, p, p, p]
     lib.km_quant_rows_i8.argtypes = [p, i64, i64, i64, i64, i32, p, p, p, p]
     lib.km_gemm_mx.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_gemm_fp8_tensor.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_gemm_fp8_rows.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
-    lib.km_gemm_fp8_blocks.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
+    lib.km_gemm_fp8_blocks.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_gemm_i8_rows.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_wo_gemm_fwd.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_wo_gemm_dgrad.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
@@ -232,24 +232,31 @@ def quant_rows(x: Tensor) -> tuple[Tensor, Tensor]:
     return q.view(E4M3), s
 
 
-def quant_blocks(x: Tensor, role: str = "act") -> tuple[Tensor, Tensor]:
+def quant_blocks(x: Tensor, role: str = "act", natural: bool = True, kmajor: bool = False):
     """`(q e4m3 [rows, K], scale fp32)` under the block recipe; any strides, K % 128 == 0.
-    `role="act"`: one scale per row and 128 columns, `[rows, K/128]`; `role="weight"`: one per
-    128 x 128 block, `[ceil(rows/128), K/128]`."""
+    `role="act"`: one scale per row and 128 columns, `[rows, K/128]`; with `kmajor` its
+    `[K/128, rows]` copy (the layout the GEMM reads fastest) is appended, and `natural=False`
+    returns None in place of the natural scales. `role="weight"`: one scale per 128 x 128 block,
+    `[ceil(rows/128), K/128]`."""
     if x.dim() != 2:
         raise ValueError(f"fp8 operand must be 2-D, got {tuple(x.shape)}")
     if role not in ("act", "weight"):
         raise ValueError(f"fp8 role {role!r} not in ('act', 'weight')")
+    if role == "weight" and (kmajor or not natural):
+        raise ValueError("weight blocks have the one scale layout")
+    if not (natural or kmajor):
+        raise ValueError("quant_blocks: ask for at least one scale layout")
     rows, k = x.shape
     if k % BLOCK:
         raise ValueError(f"fp8 block: K={k} is not a multiple of {BLOCK}")
     _on_gpu(x)
     q = torch.empty(rows, k, device=x.device, dtype=torch.uint8)
     srows = rows if role == "act" else -(-rows // BLOCK)
-    s = torch.empty(srows, k // BLOCK, device=x.device, dtype=torch.float32)
+    s = torch.empty(srows, k // BLOCK, device=x.device, dtype=torch.float32) if natural else None
+    st = torch.empty(k // BLOCK, rows, device=x.device, dtype=torch.float32) if kmajor else None
     with torch.cuda.device(x.device):
-        _check(load().km_quant_blocks(x.data_ptr(), rows, k, x.stride(0), x.stride(1), _dtype_code(x.dtype), ROLE_ACT if role == "act" else ROLE_WEIGHT, q.data_ptr(), s.data_ptr(), _stream(x)))
-    return q.view(E4M3), s
+        _check(load().km_quant_blocks(x.data_ptr(), rows, k, x.stride(0), x.stride(1), _dtype_code(x.dtype), ROLE_ACT if role == "act" else ROLE_WEIGHT, q.data_ptr(), None if s is None else s.data_ptr(), None if st is None else st.data_ptr(), _stream(x)))
+    return (q.view(E4M3), s, st) if kmajor else (q.view(E4M3), s)
 
 
 def quant_rows_i8(x: Tensor, col_scale: Tensor | None = None) -> tuple[Tensor, Tensor]:
@@ -352,19 +359,20 @@ def gemm_fp8_rows(a: Tensor, sa: Tensor, b: Tensor, sb: Tensor, bias: Tensor | N
     return c
 
 
-def gemm_fp8_blocks(a: Tensor, sa: Tensor, b: Tensor, sb: Tensor, bias: Tensor | None, out_dtype: torch.dtype, config: int = 0) -> Tensor:
-    """`sum_kb (a_kb b_kb^T) * sa[:, kb, None] * sb[n // 128, kb] + bias`; sa `[M, K/128]`, sb
-    `[ceil(N/128), K/128]` fp32 device tensors (the block recipe's activation and weight scales)."""
+def gemm_fp8_blocks(a: Tensor, sa: Tensor, b: Tensor, sb: Tensor, bias: Tensor | None, out_dtype: torch.dtype, config: int = 0, kmajor: bool = False) -> Tensor:
+    """`sum_kb (a_kb b_kb^T) * sa[:, kb, None] * sb[n // 128, kb] + bias`; sa `[M, K/128]` (with
+    `kmajor`: its `[K/128, M]` copy from `quant_blocks(kmajor=True)`), sb `[ceil(N/128), K/128]`
+    fp32 device tensors (the block recipe's activation and weight scales)."""
     a, b, bias, c, m, n, k = _gemm_operands(a, b, bias, out_dtype)
     if k % BLOCK:
         raise ValueError(f"fp8 block: K={k} is not a multiple of {BLOCK}")
-    want = ((m, k // BLOCK), (-(-n // BLOCK), k // BLOCK))
+    want = ((k // BLOCK, m) if kmajor else (m, k // BLOCK), (-(-n // BLOCK), k // BLOCK))
     if (tuple(sa.shape), tuple(sb.shape)) != want or sa.dtype != torch.float32 or sb.dtype != torch.float32:
         raise ValueError(f"block scales must be fp32 {want[0]} and {want[1]}, got {tuple(sa.shape)} {sa.dtype} and {tuple(sb.shape)} {sb.dtype}")
     _on_gpu(a, sa, sb)
     sa, sb = sa.contiguous(), sb.contiguous()
     with torch.cuda.device(a.device):
-        _check(load().km_gemm_fp8_blocks(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), None if bias is None else bias.data_ptr(), c.data_ptr(), m, n, k, _dtype_code(out_dtype), config, _stream(a)))
+        _check(load().km_gemm_fp8_blocks(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), None if bias is None else bias.data_ptr(), c.data_ptr(), m, n, k, _dtype_code(out_dtype), SCALES_KMAJOR if kmajor else SCALES_ROWMAJOR, config, _stream(a)))
     return c
 
 

@@ -38,6 +38,13 @@ def check(x_cpu, role, view=lambda t: t):
     assert q.shape == rq.shape and s.shape == rs.shape and q.is_contiguous() and s.is_contiguous()
     assert torch.equal(s.cpu().view(torch.int32), rs.view(torch.int32)), f"{role}: scale bits"
     assert torch.equal(u8(q).cpu(), u8(rq)), f"{role}: code bytes"
+    if role == "act":
+        # the K-major copy of the scales the GEMM reads: same numbers, transposed; alone or with the natural ones
+        q2, s2, st = native.quant_blocks(view(x_cpu.cuda()), role, kmajor=True)
+        q3, none, st3 = native.quant_blocks(view(x_cpu.cuda()), role, natural=False, kmajor=True)
+        assert none is None and st.shape == (rs.shape[1], rs.shape[0]) and st.is_contiguous()
+        assert torch.equal(st.view(torch.int32), s.t().view(torch.int32)) and torch.equal(st3.view(torch.int32), st.view(torch.int32))
+        assert torch.equal(u8(q2), u8(q)) and torch.equal(u8(q3), u8(q)) and torch.equal(s2.view(torch.int32), s.view(torch.int32))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -139,6 +146,8 @@ def test_block_argument_errors():
         native.quant_blocks(x.bfloat16()[:, :200], "act")
     with pytest.raises(ValueError):
         native.quant_blocks(x.bfloat16(), "bias")
+    with pytest.raises(ValueError):
+        native.quant_blocks(x.bfloat16(), "weight", kmajor=True)
     q, s = native.quant_blocks(x.bfloat16()[:0], "weight")
     assert q.shape == (0, 256) and s.shape == (0, 2)
     a = torch.zeros(8, 256, device="cuda").to(torch.float8_e4m3fn)
@@ -162,19 +171,27 @@ def gemm_operands(m, n, k, dtype, seed=0, spread=True):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("m,n,k", [(200, 384, 256), (1, 256, 512), (1000, 512, 384), (513, 200, 1024), (256, 256, 128), (130, 136, 640)])
+@pytest.mark.parametrize("m,n,k", [(200, 384, 256), (1, 256, 512), (1000, 512, 384), (513, 200, 1024), (256, 256, 128), (130, 136, 640), (384, 128, 896)])
 def test_block_gemm_against_fp64(dtype, m, n, k):
     x, w, bias = gemm_operands(m, n, k, dtype)
     xq, xs = formats.quantize(x, "block", "act")
     wq, ws = formats.quantize(w, "block", "weight")
     truth = linear.exact64(xq, xs, "block") @ linear.exact64(wq, ws, "block").T + bias.double()
     eager = linear.fp8_forward(x, wq, ws, None, bias, "block")
-    y = native.gemm_fp8_blocks(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), bias.cuda(), dtype, 0)
-    assert y.shape == (m, n) and y.dtype == dtype
-    assert_no_regression(y.cpu(), eager, truth, f"block {m}x{n}x{k}")
-    assert rel_l2(y.cpu(), truth) <= REL_L2[dtype]
-    y0 = native.gemm_fp8_blocks(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), None, dtype, 0)
-    assert rel_l2(y0.cpu(), truth - bias.double()) <= REL_L2[dtype]
+    n_cfg = len(native.configs(native.KERNEL_GEMM_BLOCKS))
+    assert n_cfg >= 2
+    for cfg in range(n_cfg):
+        y = native.gemm_fp8_blocks(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), bias.cuda(), dtype, cfg)
+        assert y.shape == (m, n) and y.dtype == dtype
+        assert_no_regression(y.cpu(), eager, truth, f"block cfg{cfg} {m}x{n}x{k}")
+        assert rel_l2(y.cpu(), truth) <= REL_L2[dtype]
+        y0 = native.gemm_fp8_blocks(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), None, dtype, cfg)
+        assert rel_l2(y0.cpu(), truth - bias.double()) <= REL_L2[dtype]
+        yk = native.gemm_fp8_blocks(xq.cuda(), xs.t().contiguous().cuda(), wq.cuda(), ws.cuda(), bias.cuda(), dtype, cfg, kmajor=True)
+        assert torch.equal(yk, y), "K-major activation scales"
+        if cfg:
+            assert torch.equal(y, first), "tile configurations add the same blocks in the same order"
+        first = y
 
 
 def test_block_gemm_uses_every_scale():
@@ -214,8 +231,8 @@ def test_block_gemm_deep_k_accumulates_in_fp32():
         worse = [s for s, slack in (("abs_mean", 1.01), ("rel_mean", 1.10)) if got[s] > slack * eager[s]]
         assert not worse, (worse, got, eager)
 
-    y = native.gemm_fp8_blocks(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), None, torch.bfloat16)
-    no_worse(y.cpu())
+    for cfg in range(len(native.configs(native.KERNEL_GEMM_BLOCKS))):
+        no_worse(native.gemm_fp8_blocks(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), None, torch.bfloat16, cfg).cpu())
     lossy = torch.zeros(m, n, dtype=torch.bfloat16)
     for kb in range(k // 128):
         sl = slice(kb * 128, (kb + 1) * 128)
