@@ -9,6 +9,7 @@ from kohakumosstrainer_amd.quant.convert import (
     quantize_model,
     quantize_torch_linears,
 )
+from kohakumosstrainer_amd.quant.stored import attach_stored, load_quantized, quantized_state, read_record, save_quantized
 from kohakumosstrainer_amd.quant.weights import QuantWeight, dequantize, quantize
 
 __all__ = [
@@ -17,9 +18,14 @@ __all__ = [
     "QuantLinear",
     "QuantWeight",
     "attach_compute",
+    "attach_stored",
     "default_filter",
     "dequantize",
+    "load_quantized",
     "quantize",
     "quantize_model",
     "quantize_torch_linears",
+    "quantized_state",
+    "read_record",
+    "save_quantized",
 ]

@@ -1,0 +1,116 @@
+"""The pre-quantized checkpoint layout (`quant.stored`, reference
+`src/kohakumoss/quant/stored.py:16-94`): record and key names, a save / load round trip that
+never materialises a 16-bit weight, and the errors. Host only (the eager backend)."""
+
+import json
+
+import pytest
+import torch
+from torch import nn
+
+from kohakumosstrainer_amd.model.linear import MossLinear
+from kohakumosstrainer_amd.quant import stored
+from kohakumosstrainer_amd.quant.compute import ComputeWeight
+
+
+class Tiny(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.a = MossLinear(256, 128, bias=True)
+        self.b = MossLinear(128, 256, bias=False)
+        self.small = MossLinear(128, 8)
+        self.norm = nn.LayerNorm(8)
+        for lin in (self.a, self.b, self.small):
+            lin.init_weights(0.05)   # MossLinear leaves its parameters unset until told
+            if lin.bias is not None:
+                nn.init.normal_(lin.bias, std=0.1)
+
+    def forward(self, x):
+        return self.norm(self.small(self.b(self.a(x))[..., :128]))
+
+
+def quantized_model(recipe, seed=0):
+    torch.manual_seed(seed)
+    m = Tiny()
+    for name in ("a", "b"):
+        lin = getattr(m, name)
+        lin.set_base(ComputeWeight.from_weight(lin.weight.detach(), recipe))
+    return m
+
+
+@pytest.mark.parametrize("recipe", ("mx", "row", "tensor", "block"))
+def test_state_layout_and_record(recipe):
+    m = quantized_model(recipe)
+    keys = ["a.weight", "a.bias", "b.weight", "small.weight", "small.bias", "norm.weight", "norm.bias"]
+    state, meta = stored.quantized_state(m, keys, torch.bfloat16)
+    record = json.loads(meta[stored.FP8_KEY])
+    assert record == {"recipe": recipe, "layers": ["a", "b"]}
+    assert stored.stored_keys(record) == ({"a.weight", "b.weight"}, {"a.weight_scale", "b.weight_scale"})
+    assert state["a.weight"].dtype == torch.float8_e4m3fn and state["a.weight"].shape == (128, 256)
+    assert torch.equal(state["a.weight"].view(torch.uint8), m.a.base.q.view(torch.uint8))
+    assert torch.equal(state["b.weight_scale"], m.b.base.scale)
+    assert state["small.weight"].dtype == torch.bfloat16 and state["norm.bias"].dtype == torch.bfloat16
+    assert set(state) == set(keys) | {"a.weight_scale", "b.weight_scale"}
+
+
+def test_one_recipe_per_checkpoint_and_folded_models_refuse():
+    m = quantized_model("mx")
+    m.b.set_base(ComputeWeight.from_weight(torch.randn(256, 128), "row"))
+    with pytest.raises(ValueError, match="one fp8 recipe"):
+        stored.quantized_state(m, ["a.weight"], torch.bfloat16)
+    m = quantized_model("mx")
+    m.fold_scales = {"x": 1.0}
+    with pytest.raises(ValueError, match="folded"):
+        stored.quantized_state(m, ["a.weight"], torch.bfloat16)
+
+
+@pytest.mark.parametrize("recipe", ("mx", "row", "block"))
+def test_save_load_round_trip(tmp_path, recipe):
+    m = quantized_model(recipe, seed=1)
+    path = tmp_path / "model.safetensors"
+    record = stored.save_quantized(m, path, torch.float32)
+    assert stored.read_record(path) == record == {"recipe": recipe, "layers": ["a", "b"]}
+    assert stored.read_record(tmp_path / "absent.safetensors") is None
+    fresh = Tiny()
+    n = stored.load_quantized(fresh, path, "cpu", torch.float32)
+    assert n == 2
+    for name in ("a", "b"):
+        lin, src = getattr(fresh, name), getattr(m, name)
+        assert isinstance(lin.base, ComputeWeight) and lin.base.recipe == recipe
+        assert lin.weight.numel() == 0, "no dense copy of a stored layer is kept"
+        assert torch.equal(lin.base.q.view(torch.uint8), src.base.q.view(torch.uint8))
+        assert torch.equal(lin.base.scale, src.base.scale)
+    assert torch.equal(fresh.small.weight, m.small.weight) and torch.equal(fresh.a.bias, m.a.bias)
+    x = torch.randn(5, 256)
+    assert torch.equal(fresh(x), m(x))
+
+
+def test_plain_file_loads_without_a_record(tmp_path):
+    from safetensors.torch import save_file
+
+    torch.manual_seed(2)
+    m = Tiny()
+    path = tmp_path / "plain.safetensors"
+    save_file({k: v.contiguous() for k, v in m.state_dict().items()}, str(path))
+    assert stored.read_record(path) is None
+    fresh = Tiny()
+    assert stored.load_quantized(fresh, path, "cpu", torch.float32) == 0
+    assert torch.equal(fresh.a.weight, m.a.weight)
+
+
+def test_record_naming_absent_tensors_or_wrong_shapes_fails(tmp_path):
+    from safetensors.torch import save_file
+
+    m = quantized_model("row")
+    state, meta = stored.quantized_state(m, ["a.weight", "a.bias", "b.weight"], torch.float32)
+    as_bytes = {k: (v.view(torch.uint8) if v.dtype == torch.float8_e4m3fn else v) for k, v in state.items()}
+    broken = dict(as_bytes)
+    del broken["b.weight_scale"]
+    save_file(broken, str(tmp_path / "lacks.safetensors"), metadata=meta)
+    with pytest.raises(KeyError):
+        stored.load_quantized(Tiny(), tmp_path / "lacks.safetensors", "cpu", torch.float32)
+    wrong = dict(as_bytes)
+    wrong["a.weight"] = wrong["a.weight"][:64].contiguous()
+    save_file(wrong, str(tmp_path / "shape.safetensors"), metadata=meta)
+    with pytest.raises(ValueError, match="stored codes"):
+        stored.load_quantized(Tiny(), tmp_path / "shape.safetensors", "cpu", torch.float32)
