@@ -1,0 +1,215 @@
+// One-launch MXFP8 linear for short M on gfx950: C = Q(x) B^T (+ bias) with x [M,K] bf16 / fp16
+// quantized to MXFP8 inside the K loop (E8M0 exponent per 32 columns, e4m3 codes: the same
+// arithmetic as the row-wise quantizer kernel, so the codes are the ones km_quant_mx writes) and
+// B [N,K] e4m3 with its MFMA-packed E8M0 scales.
+// Replaces the reference's Triton _fused_mx_kernel / fused_mx_mm
+// (src/kohakumoss_kernels/backends/triton/fp8/fused.py:98-120,182-194): at M <= 256 the
+// reference's linear is bound by launches, not by the MMA, and one launch replaces two.
+//
+// Shape of the kernel. At short M the job is to stream the weight once, so there is no LDS
+// staging and no barrier in the K loop: a workgroup owns 16*TM tokens x 32 output columns and
+// its four wavefronts split K (wavefront w takes K steps w, w+4, ...), each loading its MFMA
+// fragments straight from global memory in the MFMA's own layout (lane l: row l%16, K bytes
+// [16g, 16g+16) and [64+16g, 64+16g+16) with g = l/16), one to three steps ahead in registers. N/32
+// workgroups (288 at N = 9216) keep every compute unit streaming. A 32-column block of x lies in
+// two lanes (g and g^1); they share their 16-bit abs-max with one cross-lane exchange, and a
+// second one hands each lane the exponent byte the MFMA expects from it (lane g supplies block g).
+// The four partial sums of a workgroup meet in LDS at the end.
+#include <stdio.h>
+
+#include "km_gemm_common.h"
+#include "km_quant_common.h"
+
+namespace km {
+
+constexpr int kFusedBN = 32;
+constexpr int kFusedMaxTM = 4;
+
+// The quantizer kernels convert with MODE.FP16_OVFL set (out-of-range values saturate at +-448).
+// Here the mode stays clear, because the same wavefront's MFMAs would read the e4m3 NaN codes as
+// numbers under it. A finite block never leaves the e4m3 range (its exponent is chosen so that
+// amax * 2^-e <= 448), so only the non-finite inputs themselves need the codes the saturating
+// conversion and the reference give them: infinity -> +-448 (0x7E), NaN -> 0x7F, sign kept.
+template <int DT>
+__device__ __forceinline__ uint32_t nonfinite_fix(uint32_t codes, uint32_t h, int shift) {
+  const uint32_t a0 = h & 0x7FFFu, a1 = (h >> 16) & 0x7FFFu;
+  if (a0 >= inf16<DT>()) codes = (codes & ~(0xFFu << shift)) | (((a0 > inf16<DT>() ? 0x7Fu : 0x7Eu) | ((h >> 8) & 0x80u)) << shift);
+  if (a1 >= inf16<DT>()) codes = (codes & ~(0xFF00u << shift)) | (((a1 > inf16<DT>() ? 0x7Fu : 0x7Eu) | ((h >> 24) & 0x80u)) << (shift + 8));
+  return codes;
+}
+
+template <int DT, int OUT, int TM>
+__global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __restrict__ X, int64_t ldx, const uint8_t* __restrict__ B,
+                                                            const uint8_t* __restrict__ Bs, const uint16_t* __restrict__ bias,
+                                                            uint16_t* __restrict__ C, int M, int N, int K) {
+  constexpr int TN = kFusedBN / 16;
+  __shared__ float4 partial[4][TM * TN][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r16 = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * kFusedBN, m0 = blockIdx.y * (16 * TM);
+  const int nk = K / kStepBytes;
+  const int row_groups = (N + 127) >> 7;
+
+  struct Slab {
+    uint4 a[TM][4];   // x: elements [16g, 16g+8), [16g+8, 16g+16), [64+16g, +8), [64+16g+8, +8)
+    uint4 b[TN][2];   // codes: bytes [16g, 16g+16), [64+16g, 64+16g+16)
+    uint2 bs;         // packed scale bytes of the eight 16-row tiles of this row group, block g
+  };
+  auto load = [&](Slab& s, int ks) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      const int m = m0 + j * 16 + r16;
+      const uint4* p = reinterpret_cast<const uint4*>(X + (int64_t)m * ldx + ks * kStepBytes + 16 * g);
+      const bool live = m < M;
+      s.a[j][0] = live ? p[0] : make_uint4(0, 0, 0, 0);
+      s.a[j][1] = live ? p[1] : make_uint4(0, 0, 0, 0);
+      s.a[j][2] = live ? p[8] : make_uint4(0, 0, 0, 0);
+      s.a[j][3] = live ? p[9] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+      const uint4* p = reinterpret_cast<const uint4*>(B + (int64_t)(n0 + t * 16 + r16) * K + ks * kStepBytes + 16 * g);
+      s.b[t][0] = p[0];
+      s.b[t][1] = p[4];
+    }
+    s.bs = *reinterpret_cast<const uint2*>(Bs + (((int64_t)ks * row_groups + (n0 >> 7)) * 16 + r16) * 32 + 8 * g);
+  };
+
+  v4f acc[TN][TM];
+#pragma unroll
+  for (int t = 0; t < TN; ++t)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  auto compute = [&](const Slab& s) __attribute__((always_inline)) {
+    const uint64_t bs64 = ((uint64_t)s.bs.y << 32 | s.bs.x) >> (((n0 & 127) >> 4) * 8);
+    v8i wf[TN];
+    int wscale[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+      wf[t] = v8i{(int)s.b[t][0].x, (int)s.b[t][0].y, (int)s.b[t][0].z, (int)s.b[t][0].w, (int)s.b[t][1].x, (int)s.b[t][1].y, (int)s.b[t][1].z, (int)s.b[t][1].w};
+      wscale[t] = (int)((bs64 >> (8 * t)) & 0xFFu);
+    }
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      // abs-max of this lane's two 16-element halves, then of the 32-column blocks they belong to
+      const uint32_t a0 = amax16x8(s.a[j][0]), a1 = amax16x8(s.a[j][1]), a2 = amax16x8(s.a[j][2]), a3 = amax16x8(s.a[j][3]);
+      uint32_t m_lo = a0 > a1 ? a0 : a1, m_hi = a2 > a3 ? a2 : a3;
+      const uint32_t other = (uint32_t)__shfl_xor((int)(m_lo | (m_hi << 16)), 16);
+      m_lo = (other & 0xFFFFu) > m_lo ? (other & 0xFFFFu) : m_lo;
+      m_hi = (other >> 16) > m_hi ? (other >> 16) : m_hi;
+      const uint32_t e_lo = mx_biased_exponent(widen_bits<DT>(m_lo)), e_hi = mx_biased_exponent(widen_bits<DT>(m_hi));
+      const float sc_lo = bits_f32(e_lo << 23), sc_hi = bits_f32(e_hi << 23);
+      uint32_t c[8];
+      c[0] = cvt4<DT>(s.a[j][0].x, s.a[j][0].y, sc_lo); c[1] = cvt4<DT>(s.a[j][0].z, s.a[j][0].w, sc_lo);
+      c[2] = cvt4<DT>(s.a[j][1].x, s.a[j][1].y, sc_lo); c[3] = cvt4<DT>(s.a[j][1].z, s.a[j][1].w, sc_lo);
+      c[4] = cvt4<DT>(s.a[j][2].x, s.a[j][2].y, sc_hi); c[5] = cvt4<DT>(s.a[j][2].z, s.a[j][2].w, sc_hi);
+      c[6] = cvt4<DT>(s.a[j][3].x, s.a[j][3].y, sc_hi); c[7] = cvt4<DT>(s.a[j][3].z, s.a[j][3].w, sc_hi);
+      if ((a0 | a1 | a2 | a3) >= inf16<DT>()) {  // perhaps an infinity or a NaN among this lane's elements (rare)
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          if ((h == 0 ? a0 : h == 1 ? a1 : h == 2 ? a2 : a3) >= inf16<DT>()) {
+            c[2 * h] = nonfinite_fix<DT>(nonfinite_fix<DT>(c[2 * h], s.a[j][h].x, 0), s.a[j][h].y, 16);
+            c[2 * h + 1] = nonfinite_fix<DT>(nonfinite_fix<DT>(c[2 * h + 1], s.a[j][h].z, 0), s.a[j][h].w, 16);
+          }
+        }
+      }
+      // lane g supplies the exponent of block g: blocks 0, 1 are the low halves of lanes g' = 0-1 and
+      // 2-3, blocks 2, 3 their high halves
+      const uint32_t got = (uint32_t)__shfl((int)(e_lo | (e_hi << 8)), r16 + 16 * ((g & 1) * 2));
+      const int xscale = (int)((g < 2 ? got : got >> 8) & 0xFFu);
+      const v8i xf = v8i{(int)c[0], (int)c[1], (int)c[2], (int)c[3], (int)c[4], (int)c[5], (int)c[6], (int)c[7]};
+#pragma unroll
+      for (int t = 0; t < TN; ++t)  // MFMA rows come from B (output columns n), MFMA columns from x (tokens m)
+        acc[t][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[t], xf, acc[t][j], 0, 0, 0, wscale[t], 0, xscale);
+    }
+  };
+
+  // K steps wave, wave + 4, ...: the slabs of the next DEPTH - 1 steps are in flight while this one
+  // is multiplied (a ring of register slabs, walked by a loop unrolled over the ring)
+  constexpr int DEPTH = TM == 1 ? 4 : 2;
+  Slab ring[DEPTH];
+#pragma unroll
+  for (int d = 0; d + 1 < DEPTH; ++d)
+    if (wave + 4 * d < nk) load(ring[d], wave + 4 * d);
+  int ks = wave;
+  while (ks < nk) {
+    static_for<DEPTH>([&](auto d_tag) __attribute__((always_inline)) {
+      constexpr int d = decltype(d_tag)::value;
+      if (ks < nk) {
+        const int ahead = ks + 4 * (DEPTH - 1);
+        if (ahead < nk) load(ring[(d + DEPTH - 1) % DEPTH], ahead);
+        compute(ring[d]);
+        ks += 4;
+      }
+    });
+  }
+
+#pragma unroll
+  for (int t = 0; t < TN; ++t)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) partial[wave][t * TM + j][lane] = make_float4(acc[t][j][0], acc[t][j][1], acc[t][j][2], acc[t][j][3]);
+  __syncthreads();
+  // tile i of the TM * TN is summed and stored by wavefront i % 4: lane (r16, g) holds C[m][n .. n+3]
+#pragma unroll
+  for (int i = 0; i < TM * TN; ++i) {
+    if ((i & 3) != wave) continue;
+    const int t = i / TM, j = i % TM;
+    const int m = m0 + j * 16 + r16, n = n0 + t * 16 + 4 * g;
+    if (m >= M) continue;
+    float4 v = partial[0][i][lane];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      const float4 o = partial[w][i][lane];
+      v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+    }
+    if (bias != nullptr) {
+      const uint2 braw = *reinterpret_cast<const uint2*>(bias + n);
+      v.x += unpack1<OUT>(braw.x & 0xFFFFu); v.y += unpack1<OUT>(braw.x >> 16);
+      v.z += unpack1<OUT>(braw.y & 0xFFFFu); v.w += unpack1<OUT>(braw.y >> 16);
+    }
+    *reinterpret_cast<uint2*>(C + (int64_t)m * N + n) = make_uint2(pack2<OUT>(v.x, v.y), pack2<OUT>(v.z, v.w));
+  }
+}
+
+template <int DT, int TM>
+static void launch_fused(const void* x, int64_t ldx, const void* b, const void* bs, const void* bias, void* c, int M, int N, int K,
+                         hipStream_t st) {
+  const dim3 grid((unsigned)(N / kFusedBN), (unsigned)((M + 16 * TM - 1) / (16 * TM)));
+  hipLaunchKernelGGL((gemm_mx_fused_kernel<DT, DT, TM>), grid, dim3(256), 0, st, (const uint16_t*)x, ldx, (const uint8_t*)b,
+                     (const uint8_t*)bs, (const uint16_t*)bias, (uint16_t*)c, M, N, K);
+}
+
+template <int DT>
+static void dispatch_fused(int tm, const void* x, int64_t ldx, const void* b, const void* bs, const void* bias, void* c, int M, int N,
+                           int K, hipStream_t st) {
+  switch (tm) {
+    case 1: return launch_fused<DT, 1>(x, ldx, b, bs, bias, c, M, N, K, st);
+    case 2: return launch_fused<DT, 2>(x, ldx, b, bs, bias, c, M, N, K, st);
+    case 3: return launch_fused<DT, 3>(x, ldx, b, bs, bias, c, M, N, K, st);
+    default: return launch_fused<DT, 4>(x, ldx, b, bs, bias, c, M, N, K, st);
+  }
+}
+
+}  // namespace km
+
+using namespace km;
+
+extern "C" int km_gemm_mx_fused(const void* x, int64_t stride_row, const void* b, const void* b_scale_packed, const void* bias,
+                                void* c, int64_t M, int64_t N, int64_t K, int dtype, void* stream) {
+  if (dtype != KM_BF16 && dtype != KM_F16) return km_fail(KM_ERR_ARG, "km_gemm_mx_fused: dtype must be bf16 or f16");
+  if (M < 0 || N < 0 || K <= 0 || K % kStepBytes) return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_mx_fused: K must be a positive multiple of 128");
+  if (N % kFusedBN) return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_mx_fused: N must be a multiple of 32");
+  if (M * K > 0x7FFFFFFFll || N * K > 0x7FFFFFFFll || (M + 15) / 16 > 65535ll * kFusedMaxTM) return km_fail(KM_ERR_ARG, "km_gemm_mx_fused: dimension too large");
+  if (M == 0 || N == 0) return KM_OK;
+  if (!x || !b || !b_scale_packed || !c) return km_fail(KM_ERR_ARG, "km_gemm_mx_fused: null pointer");
+  if (stride_row < K || stride_row % 8 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(b)) & 15) ||
+      (reinterpret_cast<uintptr_t>(b_scale_packed) & 7) || (reinterpret_cast<uintptr_t>(bias) & 7) || (reinterpret_cast<uintptr_t>(c) & 7))
+    return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_mx_fused: x rows and B must be 16-byte aligned, scales, bias and output 8-byte aligned");
+  const int tm = (int)((M + 15) / 16 < kFusedMaxTM ? (M + 15) / 16 : kFusedMaxTM);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == KM_BF16) dispatch_fused<KM_BF16>(tm, x, stride_row, b, b_scale_packed, bias, c, (int)M, (int)N, (int)K, st);
+  else dispatch_fused<KM_F16>(tm, x, stride_row, b, b_scale_packed, bias, c, (int)M, (int)N, (int)K, st);
+  return km_check_launch("km_gemm_mx_fused");
+}

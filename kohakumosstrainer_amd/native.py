@@ -36,6 +36,7 @@ EXPORTS = (
     "km_quant_blocks",
     "km_quant_rows_i8",
     "km_gemm_mx",
+    "km_gemm_mx_fused",
     "km_gemm_fp8_tensor",
     "km_gemm_fp8_rows",
     "km_gemm_fp8_blocks",
@@ -72,6 +73,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.km_quant_blocks.argtypes = [p, i64, i64, i64, i64, i32, i32, p, p, p, p]
     lib.km_quant_rows_i8.argtypes = [p, i64, i64, i64, i64, i32, p, p, p, p]
     lib.km_gemm_mx.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
+    lib.km_gemm_mx_fused.argtypes = [p, i64, p, p, p, p, i64, i64, i64, i32, p]
     lib.km_gemm_fp8_tensor.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_gemm_fp8_rows.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_gemm_fp8_blocks.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
@@ -333,6 +335,37 @@ def gemm_mx(a: Tensor, a_scale: Tensor, b: Tensor, b_scale: Tensor, bias: Tensor
                 c.data_ptr(), m, n, k, _dtype_code(out_dtype), SCALES_PACKED if packed else SCALES_ROWMAJOR, config, _stream(a),
             )
         )
+    return c
+
+
+FUSED_MAX_M = 32  # beyond this the redundant activation quantization costs more than the launch it saves
+
+
+def gemm_mx_fused(x: Tensor, b: Tensor, b_scale_packed: Tensor, bias: Tensor | None) -> Tensor:
+    """`Q(x) (b * 2^(b_scale-127))^T + bias` in one launch: x `[M, K]` bf16 / fp16 is quantized to
+    MXFP8 inside the GEMM (same codes as `quant_mx`), b `[N, K]` e4m3 with its MFMA-packed scales
+    (`pack_scales`); K % 128 == 0, N % 32 == 0. Meant for M up to `FUSED_MAX_M`."""
+    if x.dim() != 2 or b.dim() != 2 or x.shape[1] != b.shape[1]:
+        raise ValueError(f"operands must be [M, K] and [N, K], got {tuple(x.shape)} and {tuple(b.shape)}")
+    if b.dtype != E4M3 or b_scale_packed.dtype != torch.uint8:
+        raise ValueError("the weight must be float8_e4m3fn with uint8 packed scales")
+    dev = _on_gpu(x, b, b_scale_packed, bias)
+    m, k = x.shape
+    n = b.shape[0]
+    if k % 128 or n % 32:
+        raise ValueError(f"the fused mx linear needs K % 128 == 0 and N % 32 == 0, got K={k}, N={n}")
+    if b_scale_packed.numel() != packed_scale_bytes(n, k):
+        raise ValueError(f"packed mx scales must hold {packed_scale_bytes(n, k)} bytes, got {b_scale_packed.numel()}")
+    if x.stride(1) != 1 or x.stride(0) % 8 or x.stride(0) < k or x.data_ptr() % 16:
+        x = x.contiguous()
+    b, b_scale_packed = b.contiguous(), b_scale_packed.contiguous()
+    if bias is not None:
+        if bias.shape != (n,):
+            raise ValueError(f"bias must be [{n}], got {tuple(bias.shape)}")
+        bias = bias.to(x.dtype).contiguous()
+    c = torch.empty(m, n, device=dev, dtype=x.dtype)
+    with torch.cuda.device(dev):
+        _check(load().km_gemm_mx_fused(x.data_ptr(), x.stride(0) if m else k, b.data_ptr(), b_scale_packed.data_ptr(), None if bias is None else bias.data_ptr(), c.data_ptr(), m, n, k, _dtype_code(x.dtype), _stream(x)))
     return c
 
 

@@ -1,0 +1,112 @@
+"""The one-launch MXFP8 linear for short M (`native.gemm_mx_fused`, the counterpart of the
+reference's Triton `fused_mx_mm`, `backends/triton/fp8/fused.py:98-120`): it quantizes x inside the
+GEMM. Checked against the fp64 product of the oracle's quantized operands with the reference's
+pass rule (stated tolerance ||y - ref|| / ||ref|| <= 2e-3 for bf16, 4e-4 for fp16), against the
+two-launch path (quantizer kernel + GEMM), and bit for bit where every partial sum is exact."""
+
+import pytest
+import torch
+
+from kohakumosstrainer_amd import native
+from kohakumosstrainer_amd.kernels import registry
+from oracle import formats, linear
+from oracle.stats import assert_no_regression, rel_l2
+
+pytestmark = pytest.mark.gpu
+REL_L2 = {torch.bfloat16: 2e-3, torch.float16: 4e-4}
+
+
+def operands(m, n, k, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(m, k, generator=g) * torch.logspace(-2, 2, m)[:, None]
+    x[:, : k // 2] *= torch.logspace(-1, 1, k // 2)[None, :]
+    if m > 2:
+        x[1] = 0.0
+    w = torch.randn(n, k, generator=g) * 0.05
+    bias = (torch.randn(n, generator=g) * 0.1).to(dtype)
+    return x.to(dtype), w, bias
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+@pytest.mark.parametrize("m,n,k", [(1, 32, 128), (5, 96, 384), (16, 256, 1024), (17, 64, 640), (33, 128, 512), (48, 160, 256), (64, 256, 3072), (100, 96, 896)])
+def test_fused_mx_against_fp64_and_the_two_launch_path(dtype, m, n, k):
+    x, w, bias = operands(m, n, k, dtype, seed=m + n)
+    xq, xs = formats.quantize(x, "mx")
+    wq, ws = formats.quantize(w, "mx", "weight")
+    truth = linear.exact64(xq, xs, "mx") @ linear.exact64(wq, ws, "mx").T + bias.double()
+    eager = linear.fp8_forward(x, wq, ws, None, bias, "mx")
+    wsp = native.pack_scales(ws.cuda())
+    y = native.gemm_mx_fused(x.cuda(), wq.cuda(), wsp, bias.cuda())
+    assert y.shape == (m, n) and y.dtype == dtype
+    assert_no_regression(y.cpu(), eager, truth, f"fused mx {m}x{n}x{k}")
+    assert rel_l2(y.cpu(), truth) <= REL_L2[dtype]
+    gq, _, gsp = native.quant_mx(x.cuda(), natural=False, packed=True)
+    two = native.gemm_mx(gq, gsp, wq.cuda(), wsp, bias.cuda(), dtype, 4, packed=True)
+    assert rel_l2(y.cpu(), two.double().cpu()) <= 2 * REL_L2[dtype]
+    y0 = native.gemm_mx_fused(x.cuda(), wq.cuda(), wsp, None)
+    assert rel_l2(y0.cpu(), truth - bias.double()) <= REL_L2[dtype]
+    # rows of x not densely packed
+    wide = torch.zeros(m, k + 64, dtype=dtype, device="cuda")
+    wide[:, :k] = x.cuda()
+    assert torch.equal(native.gemm_mx_fused(wide[:, :k], wq.cuda(), wsp, bias.cuda()), y)
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+def test_fused_mx_equals_the_two_launch_path_where_sums_are_exact(dtype):
+    """Small integers in x, small-integer codes with unit scales in W: every product and partial
+    sum is an integer below 2^24, so the order of the K split cannot matter and the fused kernel
+    must give the bytes of quantizer + GEMM. A wrong exponent byte, a wrong lane pairing of the
+    32-column blocks or a misplaced K half would change them."""
+    m, n, k = 40, 96, 1024
+    g = torch.Generator().manual_seed(3)
+    x = torch.randint(-6, 7, (m, k), generator=g).float()
+    x[:, ::64] *= 32                                   # blocks of one row with different exponents
+    x[3] = 0
+    x[5, 100:132] = 0
+    w = torch.randint(-8, 9, (n, k), generator=g).float()
+    wq = w.to(torch.float8_e4m3fn)
+    ws = torch.full((n, k // 32), 127, dtype=torch.uint8)
+    ws[:, 3] = 129
+    wsp = native.pack_scales(ws.cuda())
+    xd = x.to(dtype).cuda()
+    gq, gs, gsp = native.quant_mx(xd, packed=True)
+    two = native.gemm_mx(gq, gsp, wq.cuda(), wsp, None, dtype, 4, packed=True)
+    fused = native.gemm_mx_fused(xd, wq.cuda(), wsp, None)
+    assert torch.equal(fused, two)
+    truth = linear.exact64(gq.cpu(), gs.cpu(), "mx") @ linear.exact64(wq, ws, "mx").T
+    assert torch.equal(fused.double().cpu(), truth.to(dtype).double())
+
+
+def test_fused_mx_nan_and_inf_inputs_follow_the_quantizer():
+    m, n, k = 16, 64, 256
+    x, w, _ = operands(m, n, k, torch.bfloat16, seed=9)
+    x[2, 7] = float("nan")
+    x[4, 40] = float("inf")
+    wq, ws = formats.quantize(w, "mx", "weight")
+    wsp = native.pack_scales(ws.cuda())
+    fused = native.gemm_mx_fused(x.cuda(), wq.cuda(), wsp, None)
+    gq, _, gsp = native.quant_mx(x.cuda(), natural=False, packed=True)
+    two = native.gemm_mx(gq, gsp, wq.cuda(), wsp, None, torch.bfloat16, 4, packed=True)
+    assert torch.equal(torch.isnan(fused), torch.isnan(two))
+    keep = ~torch.isnan(two)
+    assert rel_l2(fused[keep].double().cpu(), two[keep].double().cpu()) <= 4e-3
+
+
+def test_fused_mx_argument_errors_and_planner_candidate():
+    x = torch.zeros(4, 256, device="cuda", dtype=torch.bfloat16)
+    wq = torch.zeros(48, 256, device="cuda").to(torch.float8_e4m3fn)
+    with pytest.raises(ValueError):
+        native.gemm_mx_fused(x, wq, torch.zeros(native.packed_scale_bytes(48, 256), dtype=torch.uint8, device="cuda"), None)  # N % 32
+    wq = torch.zeros(64, 256, device="cuda").to(torch.float8_e4m3fn)
+    with pytest.raises(ValueError):
+        native.gemm_mx_fused(x, wq, torch.zeros(7, dtype=torch.uint8, device="cuda"), None)
+    y = native.gemm_mx_fused(x[:0], wq, torch.zeros(native.packed_scale_bytes(64, 256), dtype=torch.uint8, device="cuda"), None)
+    assert y.shape == (0, 64)
+    from kohakumosstrainer_amd.kernels.backends.hip import fp8_linear
+
+    registry.load_backends()
+    assert fp8_linear.candidates("mx", 16, 256, 256)[0]["gemm"] == "fused"
+    assert fp8_linear.candidates("mx", 32, 256, 256)[-1]["gemm"] == "fused"
+    assert not any(c["gemm"] == "fused" for c in fp8_linear.candidates("mx", 4096, 256, 256))
+    assert not any(c["gemm"] == "fused" for c in fp8_linear.candidates("mx", 16, 48, 256))
+    assert not any(c["gemm"] == "fused" for c in fp8_linear.candidates("row", 16, 256, 256))
