@@ -194,6 +194,28 @@ def other_configs(dev, reps):
         "gemm_ms": gt, "gemm_TFLOPs": flop / gt / 1e9, "gemm_config": bcfg, "gemm_configs_ms": {str(c): t for c, t in times.items()},
         "step_ms": st, "step_TFLOPs": flop / st / 1e9, "peak_TFLOPs": FP8_PEAK_TFLOPS,
     }
+    # short M (launch-bound regime): the one-launch linear that quantizes x inside the GEMM against
+    # quantizer + GEMM, bare entry points into preallocated buffers (no allocation in the timed region)
+    w_q, _, w_sp = native.quant_mx(w, natural=False, packed=True)
+    small = {}
+    for ms in (1, 16, 32):
+        xs_ = x[:ms].contiguous()
+        y_ = torch.empty(ms, n, dtype=torch.bfloat16, device=dev)
+        q_ = torch.empty(ms, k, dtype=torch.uint8, device=dev)
+        sp_ = torch.zeros(native.packed_scale_bytes(ms, k), dtype=torch.uint8, device=dev)
+        cfg_small = len(native.configs(native.KERNEL_GEMM_MX)) - 1  # the 64-row tile
+
+        def fused_call():
+            lib.km_gemm_mx_fused(xs_.data_ptr(), k, w_q.data_ptr(), w_sp.data_ptr(), None, y_.data_ptr(), ms, n, k, native.KM_BF16, stream)
+
+        def two_calls():
+            lib.km_quant_mx(xs_.data_ptr(), ms, k, k, 1, native.KM_BF16, q_.data_ptr(), None, sp_.data_ptr(), stream)
+            lib.km_gemm_mx(q_.data_ptr(), sp_.data_ptr(), w_q.data_ptr(), w_sp.data_ptr(), None, y_.data_ptr(), ms, n, k, native.KM_BF16, native.SCALES_PACKED, cfg_small, stream)
+
+        fused_call()
+        two_calls()
+        small[f"M{ms}"] = {"fused_us": event_ms(fused_call, reps) * 1e3, "quantizer_plus_gemm_us": event_ms(two_calls, reps) * 1e3}
+    out["mx_short_M_K3072_N9216"] = {**small, "weight_MB": n * k / 1e6, "note": "one launch (x quantized inside the GEMM) vs two; the weight streams once either way"}
     # int8 compute linear (per-row int8 activations, int8 MFMA GEMM, int32 accumulation), same shape
     w_scale = (w.float().abs().amax(1).clamp_min(1e-12) / 127.0)
     w8 = torch.round(w.float() / w_scale[:, None]).clamp_(-127, 127).to(torch.int8)
