@@ -224,6 +224,43 @@ def test_block_recipe_layouts():
     assert sa[129, 0].item() == ind.fp32_scale(np.abs(row.numpy()).max())
 
 
+def test_block_recipe_every_block_matches_the_definition():
+    """Both roles, block by block in numpy: scale = RN(max(amax, 1e-12) / 448), codes = nearest e4m3
+    of RN(x / scale); a ragged row count pads the weight blocks with zeros. Scales taken over the
+    wrong extent (a whole row, 32 columns, 128 x 256) must fail."""
+    x = edge_operand(rows=300, k=384, seed=11)
+    xn = x.numpy()
+    qa, sa = formats.quantize(x, "block", "act")
+    qw, sw = formats.quantize(x, "block", "weight")
+    assert sa.shape == (300, 3) and sw.shape == (3, 3)
+    for kb in range(3):
+        cols = slice(kb * 128, kb * 128 + 128)
+        want = ind.fp32_scale(np.abs(xn[:, cols]).max(axis=1))
+        assert np.array_equal(sa[:, kb].numpy(), want)
+        assert np.array_equal(u8(qa[:, cols]), ind.nearest_e4m3((xn[:, cols] / want[:, None]).astype(np.float32)))
+        for rb in range(3):
+            rows = slice(rb * 128, min(rb * 128 + 128, 300))
+            ws = ind.fp32_scale(np.abs(xn[rows, cols]).max())
+            assert sw[rb, kb].item() == ws
+            assert np.array_equal(u8(qw[rows, cols]), ind.nearest_e4m3((xn[rows, cols] / ws).astype(np.float32)))
+
+    def per_row():
+        s_row = ind.fp32_scale(np.abs(xn).max(axis=1))
+        assert np.array_equal(u8(qa), ind.nearest_e4m3((xn / s_row[:, None]).astype(np.float32)))
+
+    def per_32():
+        s32 = ind.fp32_scale(np.abs(xn.reshape(300, 12, 32)).max(axis=2))
+        assert np.array_equal(u8(qa), ind.nearest_e4m3((xn.reshape(300, 12, 32) / s32[..., None]).astype(np.float32)).reshape(300, 384))
+
+    def wide_weight_block():
+        ws = ind.fp32_scale(np.abs(xn[:128, :256]).max())
+        assert np.array_equal(u8(qw[:128, :256]), ind.nearest_e4m3((xn[:128, :256] / ws).astype(np.float32)))
+
+    must_fail(per_row, "block scales taken per row")
+    must_fail(per_32, "block scales taken per 32 columns")
+    must_fail(wide_weight_block, "weight blocks 128 x 256")
+
+
 @pytest.mark.parametrize("recipe,role", [("tensor", "act"), ("row", "act"), ("mx", "act"), ("block", "act"), ("block", "weight")])
 def test_dequantize_is_exact_product_rounded_once(recipe, role):
     x = edge_operand(rows=130, k=256)
