@@ -114,6 +114,14 @@ int km_gemm_mx(const void *a, const void *a_scale, const void *b, const void *b_
 int km_gemm_mx_fused(const void *x, int64_t stride_row, const void *b, const void *b_scale_packed,
                      const void *bias, void *c, int64_t M, int64_t N, int64_t K, int dtype, void *stream);
 
+/* One-launch per-row fp8 linear for short M: C[m,n] = (Q(x) B^T)[m,n] * (s[m] * b_scale[n]) + bias[n],
+ * s[m] = max(amax of row m of x, 1e-12) / 448 and Q(x) = e4m3(clamp(x / s[m])) taken inside the
+ * kernel with the arithmetic of km_quant_rows (a prologue scans the rows for their abs-max), B [N,K]
+ * e4m3fn, b_scale [N] fp32 (16-byte aligned). Same shape constraints and use as km_gemm_mx_fused.
+ * Replaces Triton fused_row_mm (backends/triton/fp8/fused.py:35-68,152-165). */
+int km_gemm_fp8_rows_fused(const void *x, int64_t stride_row, const void *b, const float *b_scale,
+                           const void *bias, void *c, int64_t M, int64_t N, int64_t K, int dtype, void *stream);
+
 /* Per-tensor fp8 GEMM: C = (A B^T) * (*sa * *sb) + bias, sa / sb device fp32 scalars.
  * Replaces Triton scaled_mm for the tensor recipe (backends/triton/fp8/gemm.py:66-105,187-202)
  * and torch._scaled_mm (backends/triton/fp8/linear.py:121-130). K % 128 == 0. */

@@ -1,4 +1,4 @@
-// One-launch MXFP8 linear for short M on gfx950: C = Q(x) B^T (+ bias) with x [M,K] bf16 / fp16
+// One-launch fp8 linears for short M on gfx950 (mx and per-row recipes): C = Q(x) B^T (+ bias) with x [M,K] bf16 / fp16
 // quantized to MXFP8 inside the K loop (E8M0 exponent per 32 columns, e4m3 codes: the same
 // arithmetic as the row-wise quantizer kernel, so the codes are the ones km_quant_mx writes) and
 // B [N,K] e4m3 with its MFMA-packed E8M0 scales.
@@ -38,10 +38,14 @@ __device__ __forceinline__ uint32_t nonfinite_fix(uint32_t codes, uint32_t h, in
   return codes;
 }
 
-template <int DT, int OUT, int TM>
+// ROW: the per-row recipe instead of mx (reference _fused_row_kernel, fused.py:35-68): a prologue
+// takes each token row's abs-max over all of K (the wavefronts scan their own K steps, the maxima
+// meet in LDS), the loop quantizes with s[m] = max(amax, 1e-12) / 448 and the quotient of the row
+// quantizer kernel, the MFMAs run with unit scales and s[m] * wscale[n] multiplies the sum at the end.
+template <int DT, int OUT, int TM, bool ROW>
 __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __restrict__ X, int64_t ldx, const uint8_t* __restrict__ B,
-                                                            const uint8_t* __restrict__ Bs, const uint16_t* __restrict__ bias,
-                                                            uint16_t* __restrict__ C, int M, int N, int K) {
+                                                            const uint8_t* __restrict__ Bs, const float* __restrict__ wscales,
+                                                            const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N, int K) {
   constexpr int TN = kFusedBN / 16;
   __shared__ float4 partial[4][TM * TN][64];
   const int lane = threadIdx.x & 63;
@@ -73,8 +77,48 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
       s.b[t][0] = p[0];
       s.b[t][1] = p[4];
     }
-    s.bs = *reinterpret_cast<const uint2*>(Bs + (((int64_t)ks * row_groups + (n0 >> 7)) * 16 + r16) * 32 + 8 * g);
+    if constexpr (!ROW) s.bs = *reinterpret_cast<const uint2*>(Bs + (((int64_t)ks * row_groups + (n0 >> 7)) * 16 + r16) * 32 + 8 * g);
   };
+
+  // ROW: scale, its rounded reciprocal and the kind of every token row of this lane (row j * 16 + r16)
+  float s_row[TM], r_row[TM];
+  bool finite_row[TM], nan_row[TM];
+  if constexpr (ROW) {
+    __shared__ uint32_t row_amax[4][TM][16];
+    uint32_t m16[TM];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) m16[j] = 0;
+    for (int ks = wave; ks < nk; ks += 4) {
+#pragma unroll
+      for (int j = 0; j < TM; ++j) {
+        const int m = m0 + j * 16 + r16;
+        if (m < M) {
+          const uint4* p = reinterpret_cast<const uint4*>(X + (int64_t)m * ldx + ks * kStepBytes + 16 * g);
+          const uint32_t a0 = amax16x8(p[0]), a1 = amax16x8(p[1]), a2 = amax16x8(p[8]), a3 = amax16x8(p[9]);
+          const uint32_t a01 = a0 > a1 ? a0 : a1, a23 = a2 > a3 ? a2 : a3, a = a01 > a23 ? a01 : a23;
+          m16[j] = a > m16[j] ? a : m16[j];
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {  // the four lanes (g) that share a row, then the four wavefronts
+      uint32_t o = (uint32_t)__shfl_xor((int)m16[j], 16);
+      m16[j] = o > m16[j] ? o : m16[j];
+      o = (uint32_t)__shfl_xor((int)m16[j], 32);
+      m16[j] = o > m16[j] ? o : m16[j];
+      if (g == 0) row_amax[wave][j][r16] = m16[j];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      const uint32_t m01 = max(row_amax[0][j][r16], row_amax[1][j][r16]), m23 = max(row_amax[2][j][r16], row_amax[3][j][r16]);
+      const uint32_t mm = max(m01, m23);
+      s_row[j] = scale_of_amax16<DT>(mm);
+      r_row[j] = __fdiv_rn(1.0f, s_row[j]);
+      finite_row[j] = mm < inf16<DT>();
+      nan_row[j] = mm > inf16<DT>();
+    }
+  }
 
   v4f acc[TN][TM];
 #pragma unroll
@@ -83,7 +127,8 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
     for (int j = 0; j < TM; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
   auto compute = [&](const Slab& s) __attribute__((always_inline)) {
-    const uint64_t bs64 = ((uint64_t)s.bs.y << 32 | s.bs.x) >> (((n0 & 127) >> 4) * 8);
+    uint64_t bs64 = 0x7F7F7F7F7F7F7F7Full;  // ROW: unit MFMA scales
+    if constexpr (!ROW) bs64 = ((uint64_t)s.bs.y << 32 | s.bs.x) >> (((n0 & 127) >> 4) * 8);
     v8i wf[TN];
     int wscale[TN];
 #pragma unroll
@@ -93,6 +138,17 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
     }
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
+      if constexpr (ROW) {
+        const uint2 c0 = divided_codes8<DT>(s.a[j][0], s_row[j], r_row[j], finite_row[j], nan_row[j]);
+        const uint2 c1 = divided_codes8<DT>(s.a[j][1], s_row[j], r_row[j], finite_row[j], nan_row[j]);
+        const uint2 c2 = divided_codes8<DT>(s.a[j][2], s_row[j], r_row[j], finite_row[j], nan_row[j]);
+        const uint2 c3 = divided_codes8<DT>(s.a[j][3], s_row[j], r_row[j], finite_row[j], nan_row[j]);
+        const v8i xf = v8i{(int)c0.x, (int)c0.y, (int)c1.x, (int)c1.y, (int)c2.x, (int)c2.y, (int)c3.x, (int)c3.y};
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[t], xf, acc[t][j], 0, 0, 0, 0x7F, 0, 0x7F);
+        continue;
+      }
       // abs-max of this lane's two 16-element halves, then of the 32-column blocks they belong to
       const uint32_t a0 = amax16x8(s.a[j][0]), a1 = amax16x8(s.a[j][1]), a2 = amax16x8(s.a[j][2]), a3 = amax16x8(s.a[j][3]);
       uint32_t m_lo = a0 > a1 ? a0 : a1, m_hi = a2 > a3 ? a2 : a3;
@@ -164,6 +220,10 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
       const float4 o = partial[w][i][lane];
       v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
     }
+    if constexpr (ROW) {
+      const float4 cs = *reinterpret_cast<const float4*>(wscales + n);
+      v.x *= s_row[j] * cs.x; v.y *= s_row[j] * cs.y; v.z *= s_row[j] * cs.z; v.w *= s_row[j] * cs.w;
+    }
     if (bias != nullptr) {
       const uint2 braw = *reinterpret_cast<const uint2*>(bias + n);
       v.x += unpack1<OUT>(braw.x & 0xFFFFu); v.y += unpack1<OUT>(braw.x >> 16);
@@ -173,23 +233,42 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
   }
 }
 
-template <int DT, int TM>
-static void launch_fused(const void* x, int64_t ldx, const void* b, const void* bs, const void* bias, void* c, int M, int N, int K,
-                         hipStream_t st) {
+template <int DT, int TM, bool ROW>
+static void launch_fused(const void* x, int64_t ldx, const void* b, const void* bs, const float* wscales, const void* bias, void* c,
+                         int M, int N, int K, hipStream_t st) {
   const dim3 grid((unsigned)(N / kFusedBN), (unsigned)((M + 16 * TM - 1) / (16 * TM)));
-  hipLaunchKernelGGL((gemm_mx_fused_kernel<DT, DT, TM>), grid, dim3(256), 0, st, (const uint16_t*)x, ldx, (const uint8_t*)b,
-                     (const uint8_t*)bs, (const uint16_t*)bias, (uint16_t*)c, M, N, K);
+  hipLaunchKernelGGL((gemm_mx_fused_kernel<DT, DT, TM, ROW>), grid, dim3(256), 0, st, (const uint16_t*)x, ldx, (const uint8_t*)b,
+                     (const uint8_t*)bs, wscales, (const uint16_t*)bias, (uint16_t*)c, M, N, K);
 }
 
-template <int DT>
-static void dispatch_fused(int tm, const void* x, int64_t ldx, const void* b, const void* bs, const void* bias, void* c, int M, int N,
-                           int K, hipStream_t st) {
+template <int DT, bool ROW>
+static void dispatch_fused(int tm, const void* x, int64_t ldx, const void* b, const void* bs, const float* wscales, const void* bias,
+                           void* c, int M, int N, int K, hipStream_t st) {
   switch (tm) {
-    case 1: return launch_fused<DT, 1>(x, ldx, b, bs, bias, c, M, N, K, st);
-    case 2: return launch_fused<DT, 2>(x, ldx, b, bs, bias, c, M, N, K, st);
-    case 3: return launch_fused<DT, 3>(x, ldx, b, bs, bias, c, M, N, K, st);
-    default: return launch_fused<DT, 4>(x, ldx, b, bs, bias, c, M, N, K, st);
+    case 1: return launch_fused<DT, 1, ROW>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
+    case 2: return launch_fused<DT, 2, ROW>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
+    case 3: return launch_fused<DT, 3, ROW>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
+    default: return launch_fused<DT, 4, ROW>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
   }
+}
+
+static int check_fused(const char* who, const void* x, int64_t stride_row, const void* b, const void* scales, const void* bias,
+                       void* c, int64_t M, int64_t N, int64_t K, int dtype, int scale_align) {
+  static thread_local char msg[200];
+  auto fail = [&](int code, const char* what) {
+    snprintf(msg, sizeof msg, "%s: %s", who, what);
+    return km_fail(code, msg);
+  };
+  if (dtype != KM_BF16 && dtype != KM_F16) return fail(KM_ERR_ARG, "dtype must be bf16 or f16");
+  if (M < 0 || N < 0 || K <= 0 || K % kStepBytes) return fail(KM_ERR_UNSUPPORTED, "K must be a positive multiple of 128");
+  if (N % kFusedBN) return fail(KM_ERR_UNSUPPORTED, "N must be a multiple of 32");
+  if (M * K > 0x7FFFFFFFll || N * K > 0x7FFFFFFFll || (M + 15) / 16 > 65535ll * kFusedMaxTM) return fail(KM_ERR_ARG, "dimension too large");
+  if (M == 0 || N == 0) return KM_OK;
+  if (!x || !b || !scales || !c) return fail(KM_ERR_ARG, "null pointer");
+  if (stride_row < K || stride_row % 8 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(b)) & 15) ||
+      (reinterpret_cast<uintptr_t>(scales) & (scale_align - 1)) || (reinterpret_cast<uintptr_t>(bias) & 7) || (reinterpret_cast<uintptr_t>(c) & 7))
+    return fail(KM_ERR_UNSUPPORTED, "x rows and B must be 16-byte aligned, bias and output 8-byte aligned, scales 8 (mx) / 16 (row) bytes");
+  return KM_OK;
 }
 
 }  // namespace km
@@ -198,18 +277,22 @@ using namespace km;
 
 extern "C" int km_gemm_mx_fused(const void* x, int64_t stride_row, const void* b, const void* b_scale_packed, const void* bias,
                                 void* c, int64_t M, int64_t N, int64_t K, int dtype, void* stream) {
-  if (dtype != KM_BF16 && dtype != KM_F16) return km_fail(KM_ERR_ARG, "km_gemm_mx_fused: dtype must be bf16 or f16");
-  if (M < 0 || N < 0 || K <= 0 || K % kStepBytes) return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_mx_fused: K must be a positive multiple of 128");
-  if (N % kFusedBN) return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_mx_fused: N must be a multiple of 32");
-  if (M * K > 0x7FFFFFFFll || N * K > 0x7FFFFFFFll || (M + 15) / 16 > 65535ll * kFusedMaxTM) return km_fail(KM_ERR_ARG, "km_gemm_mx_fused: dimension too large");
-  if (M == 0 || N == 0) return KM_OK;
-  if (!x || !b || !b_scale_packed || !c) return km_fail(KM_ERR_ARG, "km_gemm_mx_fused: null pointer");
-  if (stride_row < K || stride_row % 8 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(b)) & 15) ||
-      (reinterpret_cast<uintptr_t>(b_scale_packed) & 7) || (reinterpret_cast<uintptr_t>(bias) & 7) || (reinterpret_cast<uintptr_t>(c) & 7))
-    return km_fail(KM_ERR_UNSUPPORTED, "km_gemm_mx_fused: x rows and B must be 16-byte aligned, scales, bias and output 8-byte aligned");
+  const int rc = check_fused("km_gemm_mx_fused", x, stride_row, b, b_scale_packed, bias, c, M, N, K, dtype, 8);
+  if (rc != KM_OK || M == 0 || N == 0) return rc;
   const int tm = (int)((M + 15) / 16 < kFusedMaxTM ? (M + 15) / 16 : kFusedMaxTM);
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == KM_BF16) dispatch_fused<KM_BF16>(tm, x, stride_row, b, b_scale_packed, bias, c, (int)M, (int)N, (int)K, st);
-  else dispatch_fused<KM_F16>(tm, x, stride_row, b, b_scale_packed, bias, c, (int)M, (int)N, (int)K, st);
+  if (dtype == KM_BF16) dispatch_fused<KM_BF16, false>(tm, x, stride_row, b, b_scale_packed, nullptr, bias, c, (int)M, (int)N, (int)K, st);
+  else dispatch_fused<KM_F16, false>(tm, x, stride_row, b, b_scale_packed, nullptr, bias, c, (int)M, (int)N, (int)K, st);
   return km_check_launch("km_gemm_mx_fused");
+}
+
+extern "C" int km_gemm_fp8_rows_fused(const void* x, int64_t stride_row, const void* b, const float* b_scale, const void* bias,
+                                      void* c, int64_t M, int64_t N, int64_t K, int dtype, void* stream) {
+  const int rc = check_fused("km_gemm_fp8_rows_fused", x, stride_row, b, b_scale, bias, c, M, N, K, dtype, 16);
+  if (rc != KM_OK || M == 0 || N == 0) return rc;
+  const int tm = (int)((M + 15) / 16 < kFusedMaxTM ? (M + 15) / 16 : kFusedMaxTM);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == KM_BF16) dispatch_fused<KM_BF16, true>(tm, x, stride_row, b, nullptr, b_scale, bias, c, (int)M, (int)N, (int)K, st);
+  else dispatch_fused<KM_F16, true>(tm, x, stride_row, b, nullptr, b_scale, bias, c, (int)M, (int)N, (int)K, st);
+  return km_check_launch("km_gemm_fp8_rows_fused");
 }

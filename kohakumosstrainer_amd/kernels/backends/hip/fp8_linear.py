@@ -34,18 +34,23 @@ tuning.on_reset(_RESOLVED.clear)
 def candidates(recipe: str, m: int, n: int | None = None, k: int | None = None) -> list[dict]:
     """GEMM paths of `recipe` for M rows, the planner's first pick first: the library's tile
     configurations (large tiles for large M: fewest bytes fetched per flop; smaller ones when M is
-    short or the grid would not fill 256 CUs) and, for `mx` at short M, the one-launch kernel
-    that quantizes x inside the GEMM (reference `fused` candidates, `linear.py:97,113`)."""
+    short or the grid would not fill 256 CUs) and, for `mx` and `row` at short M, the one-launch
+    kernel that quantizes x inside the GEMM (reference `fused` candidates, `linear.py:97,102-104,113`)."""
     kernel = {"mx": native.KERNEL_GEMM_MX, "block": native.KERNEL_GEMM_BLOCKS}.get(recipe, native.KERNEL_GEMM_FP8)
     cfgs = [{"gemm": "hip", **c} for c in native.configs(kernel)]
     limit = max(pow2(m, 16), min(c["bm"] for c in cfgs))
     fits = [c for c in cfgs if c["bm"] <= limit] or cfgs
     ranked = sorted(fits, key=lambda c: -(c["bm"] * c["bn"]) if m >= 1024 else c["bm"])
-    if recipe == "mx" and m <= native.FUSED_MAX_M and (n is None or n % 32 == 0) and (k is None or k % 128 == 0):
-        # measured at K3072 N9216: 9.5 us against 19 us (quantizer + GEMM) at M = 1, 13.6 against 20 at
-        # M = 16, even at M = 32: first pick up to 16 rows, a timed candidate up to 32
+    if recipe in ("mx", "row") and m <= native.FUSED_MAX_M and (n is None or n % 32 == 0) and (k is None or k % 128 == 0):
+        # measured at K3072 N9216, one launch against quantizer + GEMM. mx: 9.9 against 19 us at M = 1,
+        # 13.7 against 21 at M = 16, even at M = 32: first pick up to 16 rows, a timed candidate up to 32.
+        # row (a second pass over x for the row maxima, a quotient per element): 13.6 against 14.6 us at
+        # M = 1, behind from M = 16 on: only ever a timed candidate, up to 16 rows.
         fused = {"gemm": "fused", "id": -1, "bm": 16 * -(-max(m, 1) // 16), "bn": 32}
-        ranked.insert(0 if m <= 16 else len(ranked), fused)
+        if recipe == "mx":
+            ranked.insert(0 if m <= 16 else len(ranked), fused)
+        elif m <= 16:
+            ranked.append(fused)
     return ranked
 
 
@@ -73,6 +78,8 @@ def _run(cfg, recipe, a, bq, bs, baux, bias):
         aq, _, sa_t = native.quant_blocks(a, "act", natural=False, kmajor=True)
         return native.gemm_fp8_blocks(aq, sa_t, bq, bs.float(), bias, a.dtype, cfg["id"], kmajor=True)
     if recipe == "row":
+        if cfg["gemm"] == "fused":
+            return native.gemm_fp8_rows_fused(a, bq, bs.float(), bias)
         aq, sa = native.quant_rows(a)
         return native.gemm_fp8_rows(aq, sa, bq, bs.float(), bias, a.dtype, cfg["id"])
     aq, sa = native.quant_tensor(a)

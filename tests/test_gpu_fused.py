@@ -109,4 +109,70 @@ def test_fused_mx_argument_errors_and_planner_candidate():
     assert fp8_linear.candidates("mx", 32, 256, 256)[-1]["gemm"] == "fused"
     assert not any(c["gemm"] == "fused" for c in fp8_linear.candidates("mx", 4096, 256, 256))
     assert not any(c["gemm"] == "fused" for c in fp8_linear.candidates("mx", 16, 48, 256))
-    assert not any(c["gemm"] == "fused" for c in fp8_linear.candidates("row", 16, 256, 256))
+    assert fp8_linear.candidates("row", 16, 256, 256)[-1]["gemm"] == "fused"
+    assert not any(c["gemm"] == "fused" for c in fp8_linear.candidates("row", 32, 256, 256))
+    assert not any(c["gemm"] == "fused" for c in fp8_linear.candidates("block", 16, 256, 256))
+    assert not any(c["gemm"] == "fused" for c in fp8_linear.candidates("tensor", 16, 256, 256))
+
+
+# ---- per-row recipe ---------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+@pytest.mark.parametrize("m,n,k", [(1, 32, 128), (5, 96, 384), (16, 256, 1024), (17, 64, 640), (33, 128, 512), (48, 160, 256), (64, 256, 3072), (100, 96, 896)])
+def test_fused_row_against_fp64_and_the_two_launch_path(dtype, m, n, k):
+    x, w, bias = operands(m, n, k, dtype, seed=m + n + 1)
+    xq, xs = formats.quantize(x, "row")
+    wq, ws = formats.quantize(w, "row", "weight")
+    truth = linear.exact64(xq, xs, "row") @ linear.exact64(wq, ws, "row").T + bias.double()
+    eager = linear.fp8_forward(x, wq, ws, None, bias, "row")
+    y = native.gemm_fp8_rows_fused(x.cuda(), wq.cuda(), ws.cuda(), bias.cuda())
+    assert y.shape == (m, n) and y.dtype == dtype
+    assert_no_regression(y.cpu(), eager, truth, f"fused row {m}x{n}x{k}")
+    assert rel_l2(y.cpu(), truth) <= REL_L2[dtype]
+    gq, gs = native.quant_rows(x.cuda())
+    two = native.gemm_fp8_rows(gq, gs, wq.cuda(), ws.cuda(), bias.cuda(), dtype, 4)
+    assert rel_l2(y.cpu(), two.double().cpu()) <= 2 * REL_L2[dtype]
+    y0 = native.gemm_fp8_rows_fused(x.cuda(), wq.cuda(), ws.cuda(), None)
+    assert rel_l2(y0.cpu(), truth - bias.double()) <= REL_L2[dtype]
+    wide = torch.zeros(m, k + 64, dtype=dtype, device="cuda")
+    wide[:, :k] = x.cuda()
+    assert torch.equal(native.gemm_fp8_rows_fused(wide[:, :k], wq.cuda(), ws.cuda(), bias.cuda()), y)
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+def test_fused_row_equals_the_two_launch_path_where_sums_are_exact(dtype):
+    """Rows whose abs-max is 448 * 2^e have the scale 2^e exactly; with small-integer multiples of
+    it in x and small-integer codes in W every partial sum is exact, so the fused kernel must give
+    the bytes of quantizer + GEMM whatever the K split. The row maximum sits in a different K step
+    (wavefront) for every row: a prologue that missed a wavefront's share would change the scale."""
+    m, n, k = 40, 96, 1024
+    g = torch.Generator().manual_seed(5)
+    x = torch.randint(-6, 7, (m, k), generator=g).float()
+    for r in range(m):
+        x[r] *= 2.0 ** (r % 7 - 3)
+        x[r, (r * 131) % k] = 448.0 * 2.0 ** (r % 7 - 3) / 64   # amax = 7 * 2^e: s = 2^(e-6) exactly
+    x[3] = 0
+    w = torch.randint(-8, 9, (n, k), generator=g).float()
+    wq = w.to(torch.float8_e4m3fn)
+    ws = (torch.ones(n) * 0.5).float()
+    xd = x.to(dtype).cuda()
+    assert torch.equal(xd.float().cpu(), x)
+    gq, gs = native.quant_rows(xd)
+    two = native.gemm_fp8_rows(gq, gs, wq.cuda(), ws.cuda(), None, dtype, 4)
+    fused = native.gemm_fp8_rows_fused(xd, wq.cuda(), ws.cuda(), None)
+    assert torch.equal(fused, two)
+
+
+def test_fused_row_nonfinite_rows_follow_the_quantizer():
+    m, n, k = 16, 64, 256
+    x, w, _ = operands(m, n, k, torch.bfloat16, seed=9)
+    x[2, 7] = float("nan")
+    x[4, 200] = float("inf")
+    wq, ws = formats.quantize(w, "row", "weight")
+    fused = native.gemm_fp8_rows_fused(x.cuda(), wq.cuda(), ws.cuda(), None)
+    gq, gs = native.quant_rows(x.cuda())
+    two = native.gemm_fp8_rows(gq, gs, wq.cuda(), ws.cuda(), None, torch.bfloat16, 4)
+    assert torch.equal(torch.isnan(fused), torch.isnan(two))
+    keep = ~torch.isnan(two)
+    assert rel_l2(fused[keep].double().cpu(), two[keep].double().cpu()) <= 4e-3
