@@ -108,8 +108,8 @@ int km_gemm_mx(const void *a, const void *a_scale, const void *b, const void *b_
  * bf16 / fp16 (row pitch stride_row elements, unit column stride, 16-byte aligned rows) quantized
  * to MXFP8 inside the K loop with the arithmetic of km_quant_mx, B [N,K] e4m3fn, b_scale_packed its
  * MFMA-packed E8M0 scales (km_scales_pack), bias [N] and C in x's dtype. K % 128 == 0, N % 32 == 0.
- * Every workgroup quantizes its own rows of x again (N/32 times in all), so it pays only where
- * launches, not the MFMA, bound the linear: M up to about 32.
+ * Every workgroup quantizes its own rows of x again (N/64 times in all; N/32 when N % 64 != 0), so it
+ * pays only where launches, not the MFMA, bound the linear: M up to about 32.
  * Replaces Triton fused_mx_mm (backends/triton/fp8/fused.py:98-120,182-194). */
 int km_gemm_mx_fused(const void *x, int64_t stride_row, const void *b, const void *b_scale_packed,
                      const void *bias, void *c, int64_t M, int64_t N, int64_t K, int dtype, void *stream);

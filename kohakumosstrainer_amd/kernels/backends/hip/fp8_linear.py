@@ -42,11 +42,11 @@ def candidates(recipe: str, m: int, n: int | None = None, k: int | None = None) 
     fits = [c for c in cfgs if c["bm"] <= limit] or cfgs
     ranked = sorted(fits, key=lambda c: -(c["bm"] * c["bn"]) if m >= 1024 else c["bm"])
     if recipe in ("mx", "row") and m <= native.FUSED_MAX_M and (n is None or n % 32 == 0) and (k is None or k % 128 == 0):
-        # measured at K3072 N9216, one launch against quantizer + GEMM. mx: 9.9 against 19 us at M = 1,
-        # 13.7 against 21 at M = 16, even at M = 32: first pick up to 16 rows, a timed candidate up to 32.
-        # row (a second pass over x for the row maxima, a quotient per element): 13.6 against 14.6 us at
-        # M = 1, behind from M = 16 on: only ever a timed candidate, up to 16 rows.
-        fused = {"gemm": "fused", "id": -1, "bm": 16 * -(-max(m, 1) // 16), "bn": 32}
+        # measured at K3072 N9216, one launch against quantizer + GEMM. mx: 9.1 against 19 us at M = 1,
+        # 11.0 against 21 at M = 16, 15.4 against 21 at M = 32 (even at 48): first pick up to 16 rows, a
+        # timed candidate up to 32. row (a second pass over x for the row maxima, a quotient per
+        # element): 11.9 against 14.6 us at M = 1, even at M = 16: only ever a timed candidate, up to 16 rows.
+        fused = {"gemm": "fused", "id": -1, "bm": 16 * -(-max(m, 1) // 16), "bn": 64 if (n or 64) % 64 == 0 else 32}
         if recipe == "mx":
             ranked.insert(0 if m <= 16 else len(ranked), fused)
         elif m <= 16:

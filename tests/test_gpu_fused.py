@@ -28,7 +28,7 @@ def operands(m, n, k, dtype, seed=0):
 
 
 @pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
-@pytest.mark.parametrize("m,n,k", [(1, 32, 128), (5, 96, 384), (16, 256, 1024), (17, 64, 640), (33, 128, 512), (48, 160, 256), (64, 256, 3072), (100, 96, 896)])
+@pytest.mark.parametrize("m,n,k", [(1, 32, 128), (5, 96, 384), (16, 256, 1024), (17, 64, 640), (32, 192, 384), (20, 96, 256), (33, 128, 512), (48, 160, 256), (48, 192, 640), (64, 256, 3072), (100, 96, 896), (100, 128, 384)])
 def test_fused_mx_against_fp64_and_the_two_launch_path(dtype, m, n, k):
     x, w, bias = operands(m, n, k, dtype, seed=m + n)
     xq, xs = formats.quantize(x, "mx")
@@ -57,7 +57,11 @@ def test_fused_mx_equals_the_two_launch_path_where_sums_are_exact(dtype):
     sum is an integer below 2^24, so the order of the K split cannot matter and the fused kernel
     must give the bytes of quantizer + GEMM. A wrong exponent byte, a wrong lane pairing of the
     32-column blocks or a misplaced K half would change them."""
-    m, n, k = 40, 96, 1024
+    exact_case_mx(dtype, 40, 96, 1024)
+    exact_case_mx(dtype, 30, 128, 512)    # two row tiles, 64-column workgroups
+
+
+def exact_case_mx(dtype, m, n, k):
     g = torch.Generator().manual_seed(3)
     x = torch.randint(-6, 7, (m, k), generator=g).float()
     x[:, ::64] *= 32                                   # blocks of one row with different exponents
@@ -119,7 +123,7 @@ def test_fused_mx_argument_errors_and_planner_candidate():
 
 
 @pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
-@pytest.mark.parametrize("m,n,k", [(1, 32, 128), (5, 96, 384), (16, 256, 1024), (17, 64, 640), (33, 128, 512), (48, 160, 256), (64, 256, 3072), (100, 96, 896)])
+@pytest.mark.parametrize("m,n,k", [(1, 32, 128), (5, 96, 384), (16, 256, 1024), (17, 64, 640), (32, 192, 384), (20, 96, 256), (33, 128, 512), (48, 160, 256), (48, 192, 640), (64, 256, 3072), (100, 96, 896), (100, 128, 384)])
 def test_fused_row_against_fp64_and_the_two_launch_path(dtype, m, n, k):
     x, w, bias = operands(m, n, k, dtype, seed=m + n + 1)
     xq, xs = formats.quantize(x, "row")
@@ -146,7 +150,11 @@ def test_fused_row_equals_the_two_launch_path_where_sums_are_exact(dtype):
     it in x and small-integer codes in W every partial sum is exact, so the fused kernel must give
     the bytes of quantizer + GEMM whatever the K split. The row maximum sits in a different K step
     (wavefront) for every row: a prologue that missed a wavefront's share would change the scale."""
-    m, n, k = 40, 96, 1024
+    exact_case_row(dtype, 40, 96, 1024)
+    exact_case_row(dtype, 30, 128, 512)   # two row tiles, 64-column workgroups
+
+
+def exact_case_row(dtype, m, n, k):
     g = torch.Generator().manual_seed(5)
     x = torch.randint(-6, 7, (m, k), generator=g).float()
     for r in range(m):
