@@ -184,3 +184,43 @@ def test_fused_row_nonfinite_rows_follow_the_quantizer():
     assert torch.equal(torch.isnan(fused), torch.isnan(two))
     keep = ~torch.isnan(two)
     assert rel_l2(fused[keep].double().cpu(), two[keep].double().cpu()) <= 4e-3
+
+
+# ---- through the registered op ------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("recipe", ("mx", "row"))
+def test_short_m_through_the_registered_op(recipe, tmp_path, monkeypatch):
+    """`fp8_linear` at 8 rows: with timing off the planner binds its first candidate (mx: the
+    one-launch kernel); with the table on it times the one-launch kernel among the tile
+    configurations and stores a winner. Either way the result obeys the GEMM tolerance."""
+    from kohakumosstrainer_amd.kernels import tuning
+    from kohakumosstrainer_amd.kernels.backends.hip import fp8_linear
+    from kohakumosstrainer_amd.quant.compute import ComputeWeight
+
+    registry.load_backends()
+    m, n, k = 8, 256, 512
+    x, w, bias = operands(m, n, k, torch.bfloat16, seed=21)
+    xq, xs = formats.quantize(x, recipe)
+    wq, ws = formats.quantize(w.to(torch.bfloat16), recipe, "weight")
+    truth = linear.exact64(xq, xs, recipe) @ linear.exact64(wq, ws, recipe).T + bias.double()
+    monkeypatch.setenv("KOHAKUMOSS_KERNEL_CACHE", str(tmp_path))
+    try:
+        for mode in ("off", "table"):
+            tuning._tables.clear()
+            tuning.set_mode(mode)
+            tuning.reset()
+            cw = ComputeWeight.from_weight(w.to(torch.bfloat16).cuda(), recipe)
+            cw.bind(torch.bfloat16, torch.device("cuda"))
+            y = cw.linear(x.cuda(), bias.cuda())
+            assert rel_l2(y.cpu(), truth) <= REL_L2[torch.bfloat16], (recipe, mode)
+            chosen = fp8_linear._select("fwd", x.cuda(), cw.q, cw.scale, cw.aux, bias.cuda(), recipe, False)
+            if mode == "off":
+                assert chosen["gemm"] == ("fused" if recipe == "mx" else "hip")
+            else:
+                rows = list(tmp_path.rglob("fp8_fwd.json"))
+                assert len(rows) == 1 and "fused" in rows[0].read_text(), "the one-launch kernel was among the timed candidates"
+    finally:
+        tuning._tables.clear()
+        tuning.set_mode("table")
+        tuning.reset()
