@@ -122,6 +122,14 @@ int km_gemm_mx_fused(const void *x, int64_t stride_row, const void *b, const voi
 int km_gemm_fp8_rows_fused(const void *x, int64_t stride_row, const void *b, const float *b_scale,
                            const void *bias, void *c, int64_t M, int64_t N, int64_t K, int dtype, void *stream);
 
+/* One-launch block-recipe fp8 linear for short M: C[m,n] = sum over K blocks kb of (Q(x)[m,kb] . B[n,kb])
+ * * s[m,kb] * b_scale[n/128,kb] + bias[n], with s[m,kb] = max(amax of x[m, 128 kb .. 128 kb + 127], 1e-12) / 448
+ * and Q(x) = e4m3(clamp(x / s)) taken inside the kernel with the arithmetic of km_quant_blocks
+ * (KM_ROLE_ACT); B [N,K] e4m3fn, b_scale [ceil(N/128), K/128] fp32. Same shape constraints and use as
+ * km_gemm_mx_fused. Replaces Triton fused_block_mm (backends/triton/fp8/fused.py:71-95,167-179). */
+int km_gemm_fp8_blocks_fused(const void *x, int64_t stride_row, const void *b, const float *b_scale,
+                             const void *bias, void *c, int64_t M, int64_t N, int64_t K, int dtype, void *stream);
+
 /* Per-tensor fp8 GEMM: C = (A B^T) * (*sa * *sb) + bias, sa / sb device fp32 scalars.
  * Replaces Triton scaled_mm for the tensor recipe (backends/triton/fp8/gemm.py:66-105,187-202)
  * and torch._scaled_mm (backends/triton/fp8/linear.py:121-130). K % 128 == 0. */

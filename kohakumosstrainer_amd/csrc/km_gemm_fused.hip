@@ -1,4 +1,4 @@
-// One-launch fp8 linears for short M on gfx950 (mx and per-row recipes): C = Q(x) B^T (+ bias) with x [M,K] bf16 / fp16
+// One-launch fp8 linears for short M on gfx950 (mx, per-row and block recipes): C = Q(x) B^T (+ bias) with x [M,K] bf16 / fp16
 // quantized to MXFP8 inside the K loop (E8M0 exponent per 32 columns, e4m3 codes: the same
 // arithmetic as the row-wise quantizer kernel, so the codes are the ones km_quant_mx writes) and
 // B [N,K] e4m3 with its MFMA-packed E8M0 scales.
@@ -42,10 +42,17 @@ __device__ __forceinline__ uint32_t nonfinite_fix(uint32_t codes, uint32_t h, in
 // takes each token row's abs-max over all of K (the wavefronts scan their own K steps, the maxima
 // meet in LDS), the loop quantizes with s[m] = max(amax, 1e-12) / 448 and the quotient of the row
 // quantizer kernel, the MFMAs run with unit scales and s[m] * wscale[n] multiplies the sum at the end.
-template <int DT, int OUT, int TM, int TN, bool ROW>
+// MODE kFusedBlock: the block recipe (reference _fused_block_kernel, fused.py:71-95): every K step is
+// one 128-column block, so a row's abs-max over the step is its block's (the four lanes that share
+// the row exchange theirs), the step's MFMA sum starts from zero and is promoted with
+// s[m, kb] * wscales[n / 128, kb]; wscales is then the [ceil(N/128), K/128] weight block scale matrix.
+constexpr int kFusedMx = 0, kFusedRow = 1, kFusedBlock = 2;
+
+template <int DT, int OUT, int TM, int TN, int MODE>
 __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __restrict__ X, int64_t ldx, const uint8_t* __restrict__ B,
                                                             const uint8_t* __restrict__ Bs, const float* __restrict__ wscales,
                                                             const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N, int K) {
+  constexpr bool ROW = MODE == kFusedRow, BLOCK = MODE == kFusedBlock;
   constexpr int BN = 16 * TN;  // 32 output columns, or 64: half as many workgroups quantize x again
   __shared__ float4 partial[4][TM * TN][64];
   const int lane = threadIdx.x & 63;
@@ -58,7 +65,8 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
   struct Slab {
     uint4 a[TM][4];   // x: elements [16g, 16g+8), [16g+8, 16g+16), [64+16g, +8), [64+16g+8, +8)
     uint4 b[TN][2];   // codes: bytes [16g, 16g+16), [64+16g, 64+16g+16)
-    uint2 bs;         // packed scale bytes of the eight 16-row tiles of this row group, block g
+    uint2 bs;         // mx: packed scale bytes of the eight 16-row tiles of this row group, block g
+    float wb;         // block recipe: the scale of this step's 128 x 128 weight block
   };
   auto load = [&](Slab& s, int ks) __attribute__((always_inline)) {
 #pragma unroll
@@ -77,7 +85,8 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
       s.b[t][0] = p[0];
       s.b[t][1] = p[4];
     }
-    if constexpr (!ROW) s.bs = *reinterpret_cast<const uint2*>(Bs + (((int64_t)ks * row_groups + (n0 >> 7)) * 16 + r16) * 32 + 8 * g);
+    if constexpr (MODE == kFusedMx) s.bs = *reinterpret_cast<const uint2*>(Bs + (((int64_t)ks * row_groups + (n0 >> 7)) * 16 + r16) * 32 + 8 * g);
+    if constexpr (BLOCK) s.wb = wscales[(int64_t)(n0 >> 7) * nk + ks];
   };
 
   // ROW: scale, its rounded reciprocal and the kind of every token row of this lane (row j * 16 + r16)
@@ -127,8 +136,8 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
     for (int j = 0; j < TM; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
   auto compute = [&](const Slab& s) __attribute__((always_inline)) {
-    uint64_t bs64 = 0x7F7F7F7F7F7F7F7Full;  // ROW: unit MFMA scales
-    if constexpr (!ROW) bs64 = ((uint64_t)s.bs.y << 32 | s.bs.x) >> (((n0 & 127) >> 4) * 8);
+    uint64_t bs64 = 0x7F7F7F7F7F7F7F7Full;  // row and block recipes: unit MFMA scales
+    if constexpr (MODE == kFusedMx) bs64 = ((uint64_t)s.bs.y << 32 | s.bs.x) >> (((n0 & 127) >> 4) * 8);
     v8i wf[TN];
     int wscale[TN];
 #pragma unroll
@@ -138,6 +147,28 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
     }
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
+      if constexpr (BLOCK) {
+        const uint32_t a0 = amax16x8(s.a[j][0]), a1 = amax16x8(s.a[j][1]), a2 = amax16x8(s.a[j][2]), a3 = amax16x8(s.a[j][3]);
+        const uint32_t a01 = a0 > a1 ? a0 : a1, a23 = a2 > a3 ? a2 : a3;
+        uint32_t mm = a01 > a23 ? a01 : a23;
+        uint32_t o = (uint32_t)__shfl_xor((int)mm, 16);
+        mm = o > mm ? o : mm;
+        o = (uint32_t)__shfl_xor((int)mm, 32);
+        mm = o > mm ? o : mm;
+        const float sc = scale_of_amax16<DT>(mm), rc = __fdiv_rn(1.0f, sc);
+        const bool fin = mm < inf16<DT>(), nan = mm > inf16<DT>();
+        const uint2 c0 = divided_codes8<DT>(s.a[j][0], sc, rc, fin, nan), c1 = divided_codes8<DT>(s.a[j][1], sc, rc, fin, nan);
+        const uint2 c2 = divided_codes8<DT>(s.a[j][2], sc, rc, fin, nan), c3 = divided_codes8<DT>(s.a[j][3], sc, rc, fin, nan);
+        const v8i xf = v8i{(int)c0.x, (int)c0.y, (int)c1.x, (int)c1.y, (int)c2.x, (int)c2.y, (int)c3.x, (int)c3.y};
+        const float promote = sc * s.wb;
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+          const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[t], xf, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0x7F, 0, 0x7F);
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[t][j][v] = __builtin_fmaf(part[v], promote, acc[t][j][v]);
+        }
+        continue;
+      }
       if constexpr (ROW) {
         const uint2 c0 = divided_codes8<DT>(s.a[j][0], s_row[j], r_row[j], finite_row[j], nan_row[j]);
         const uint2 c1 = divided_codes8<DT>(s.a[j][1], s_row[j], r_row[j], finite_row[j], nan_row[j]);
@@ -233,31 +264,31 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
   }
 }
 
-template <int DT, int TM, int TN, bool ROW>
+template <int DT, int TM, int TN, int MODE>
 static void launch_fused(const void* x, int64_t ldx, const void* b, const void* bs, const float* wscales, const void* bias, void* c,
                          int M, int N, int K, hipStream_t st) {
   const dim3 grid((unsigned)(N / (16 * TN)), (unsigned)((M + 16 * TM - 1) / (16 * TM)));
-  hipLaunchKernelGGL((gemm_mx_fused_kernel<DT, DT, TM, TN, ROW>), grid, dim3(256), 0, st, (const uint16_t*)x, ldx, (const uint8_t*)b,
+  hipLaunchKernelGGL((gemm_mx_fused_kernel<DT, DT, TM, TN, MODE>), grid, dim3(256), 0, st, (const uint16_t*)x, ldx, (const uint8_t*)b,
                      (const uint8_t*)bs, wscales, (const uint16_t*)bias, (uint16_t*)c, M, N, K);
 }
 
 // 64-column workgroups when N allows: half as many of them quantize x again, and the weight still
 // streams through 144 workgroups at N = 9216 (measured: 32 columns 13.7 us, 64 columns 11.2 us,
 // 128 columns 16.7 us at M = 16, K3072 N9216).
-template <int DT, bool ROW>
+template <int DT, int MODE>
 static void dispatch_fused(const void* x, int64_t ldx, const void* b, const void* bs, const float* wscales, const void* bias,
                            void* c, int M, int N, int K, hipStream_t st) {
   const int tiles = (M + 15) / 16;
   if (N % 64 == 0) {
-    if (tiles <= 1) return launch_fused<DT, 1, 4, ROW>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
-    if (tiles == 2) return launch_fused<DT, 2, 4, ROW>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
-    if (tiles == 3) return launch_fused<DT, 3, 4, ROW>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
-    return launch_fused<DT, 4, 4, ROW>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
+    if (tiles <= 1) return launch_fused<DT, 1, 4, MODE>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
+    if (tiles == 2) return launch_fused<DT, 2, 4, MODE>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
+    if (tiles == 3) return launch_fused<DT, 3, 4, MODE>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
+    return launch_fused<DT, 4, 4, MODE>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
   }
-  if (tiles <= 1) return launch_fused<DT, 1, 2, ROW>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
-  if (tiles == 2) return launch_fused<DT, 2, 2, ROW>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
-  if (tiles == 3) return launch_fused<DT, 3, 2, ROW>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
-  return launch_fused<DT, 4, 2, ROW>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
+  if (tiles <= 1) return launch_fused<DT, 1, 2, MODE>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
+  if (tiles == 2) return launch_fused<DT, 2, 2, MODE>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
+  if (tiles == 3) return launch_fused<DT, 3, 2, MODE>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
+  return launch_fused<DT, 4, 2, MODE>(x, ldx, b, bs, wscales, bias, c, M, N, K, st);
 }
 
 static int check_fused(const char* who, const void* x, int64_t stride_row, const void* b, const void* scales, const void* bias,
@@ -275,7 +306,7 @@ static int check_fused(const char* who, const void* x, int64_t stride_row, const
   if (!x || !b || !scales || !c) return fail(KM_ERR_ARG, "null pointer");
   if (stride_row < K || stride_row % 8 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(b)) & 15) ||
       (reinterpret_cast<uintptr_t>(scales) & (scale_align - 1)) || (reinterpret_cast<uintptr_t>(bias) & 7) || (reinterpret_cast<uintptr_t>(c) & 7))
-    return fail(KM_ERR_UNSUPPORTED, "x rows and B must be 16-byte aligned, bias and output 8-byte aligned, scales 8 (mx) / 16 (row) bytes");
+    return fail(KM_ERR_UNSUPPORTED, "x rows and B must be 16-byte aligned, bias and output 8-byte aligned, scales 8 (mx) / 16 (row) / 4 (block) bytes");
   return KM_OK;
 }
 
@@ -288,8 +319,8 @@ extern "C" int km_gemm_mx_fused(const void* x, int64_t stride_row, const void* b
   const int rc = check_fused("km_gemm_mx_fused", x, stride_row, b, b_scale_packed, bias, c, M, N, K, dtype, 8);
   if (rc != KM_OK || M == 0 || N == 0) return rc;
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == KM_BF16) dispatch_fused<KM_BF16, false>(x, stride_row, b, b_scale_packed, nullptr, bias, c, (int)M, (int)N, (int)K, st);
-  else dispatch_fused<KM_F16, false>(x, stride_row, b, b_scale_packed, nullptr, bias, c, (int)M, (int)N, (int)K, st);
+  if (dtype == KM_BF16) dispatch_fused<KM_BF16, kFusedMx>(x, stride_row, b, b_scale_packed, nullptr, bias, c, (int)M, (int)N, (int)K, st);
+  else dispatch_fused<KM_F16, kFusedMx>(x, stride_row, b, b_scale_packed, nullptr, bias, c, (int)M, (int)N, (int)K, st);
   return km_check_launch("km_gemm_mx_fused");
 }
 
@@ -298,7 +329,17 @@ extern "C" int km_gemm_fp8_rows_fused(const void* x, int64_t stride_row, const v
   const int rc = check_fused("km_gemm_fp8_rows_fused", x, stride_row, b, b_scale, bias, c, M, N, K, dtype, 16);
   if (rc != KM_OK || M == 0 || N == 0) return rc;
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == KM_BF16) dispatch_fused<KM_BF16, true>(x, stride_row, b, nullptr, b_scale, bias, c, (int)M, (int)N, (int)K, st);
-  else dispatch_fused<KM_F16, true>(x, stride_row, b, nullptr, b_scale, bias, c, (int)M, (int)N, (int)K, st);
+  if (dtype == KM_BF16) dispatch_fused<KM_BF16, kFusedRow>(x, stride_row, b, nullptr, b_scale, bias, c, (int)M, (int)N, (int)K, st);
+  else dispatch_fused<KM_F16, kFusedRow>(x, stride_row, b, nullptr, b_scale, bias, c, (int)M, (int)N, (int)K, st);
   return km_check_launch("km_gemm_fp8_rows_fused");
+}
+
+extern "C" int km_gemm_fp8_blocks_fused(const void* x, int64_t stride_row, const void* b, const float* b_scale, const void* bias,
+                                        void* c, int64_t M, int64_t N, int64_t K, int dtype, void* stream) {
+  const int rc = check_fused("km_gemm_fp8_blocks_fused", x, stride_row, b, b_scale, bias, c, M, N, K, dtype, 4);
+  if (rc != KM_OK || M == 0 || N == 0) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == KM_BF16) dispatch_fused<KM_BF16, kFusedBlock>(x, stride_row, b, nullptr, b_scale, bias, c, (int)M, (int)N, (int)K, st);
+  else dispatch_fused<KM_F16, kFusedBlock>(x, stride_row, b, nullptr, b_scale, bias, c, (int)M, (int)N, (int)K, st);
+  return km_check_launch("km_gemm_fp8_blocks_fused");
 }

@@ -34,20 +34,21 @@ tuning.on_reset(_RESOLVED.clear)
 def candidates(recipe: str, m: int, n: int | None = None, k: int | None = None) -> list[dict]:
     """GEMM paths of `recipe` for M rows, the planner's first pick first: the library's tile
     configurations (large tiles for large M: fewest bytes fetched per flop; smaller ones when M is
-    short or the grid would not fill 256 CUs) and, for `mx` and `row` at short M, the one-launch
+    short or the grid would not fill 256 CUs) and, for `mx`, `row` and `block` at short M, the one-launch
     kernel that quantizes x inside the GEMM (reference `fused` candidates, `linear.py:97,102-104,113`)."""
     kernel = {"mx": native.KERNEL_GEMM_MX, "block": native.KERNEL_GEMM_BLOCKS}.get(recipe, native.KERNEL_GEMM_FP8)
     cfgs = [{"gemm": "hip", **c} for c in native.configs(kernel)]
     limit = max(pow2(m, 16), min(c["bm"] for c in cfgs))
     fits = [c for c in cfgs if c["bm"] <= limit] or cfgs
     ranked = sorted(fits, key=lambda c: -(c["bm"] * c["bn"]) if m >= 1024 else c["bm"])
-    if recipe in ("mx", "row") and m <= native.FUSED_MAX_M and (n is None or n % 32 == 0) and (k is None or k % 128 == 0):
+    if recipe in ("mx", "row", "block") and m <= native.FUSED_MAX_M and (n is None or n % 32 == 0) and (k is None or k % 128 == 0):
         # measured at K3072 N9216, one launch against quantizer + GEMM. mx: 9.1 against 19 us at M = 1,
-        # 11.0 against 21 at M = 16, 15.4 against 21 at M = 32 (even at 48): first pick up to 16 rows, a
-        # timed candidate up to 32. row (a second pass over x for the row maxima, a quotient per
-        # element): 11.9 against 14.6 us at M = 1, even at M = 16: only ever a timed candidate, up to 16 rows.
+        # 11.0 against 21 at M = 16, 15.4 against 21 at M = 32 (even at 48); block: 11.9 against 21.5, 13.3
+        # against 22.7, 19.2 against 23.0: first pick up to 16 rows, a timed candidate up to 32. row (a
+        # second pass over x for the row maxima): 11.9 against 14.6 us at M = 1, even at M = 16: only
+        # ever a timed candidate, up to 16 rows.
         fused = {"gemm": "fused", "id": -1, "bm": 16 * -(-max(m, 1) // 16), "bn": 64 if (n or 64) % 64 == 0 else 32}
-        if recipe == "mx":
+        if recipe in ("mx", "block"):
             ranked.insert(0 if m <= 16 else len(ranked), fused)
         elif m <= 16:
             ranked.append(fused)
@@ -75,6 +76,8 @@ def _run(cfg, recipe, a, bq, bs, baux, bias):
         aq, _, a_packed = native.quant_mx(a, natural=False, packed=True)
         return native.gemm_mx(aq, a_packed, bq, baux, bias, a.dtype, cfg["id"], packed=True)
     if recipe == "block":
+        if cfg["gemm"] == "fused":
+            return native.gemm_fp8_blocks_fused(a, bq, bs.float(), bias)
         aq, _, sa_t = native.quant_blocks(a, "act", natural=False, kmajor=True)
         return native.gemm_fp8_blocks(aq, sa_t, bq, bs.float(), bias, a.dtype, cfg["id"], kmajor=True)
     if recipe == "row":

@@ -38,6 +38,7 @@ EXPORTS = (
     "km_gemm_mx",
     "km_gemm_mx_fused",
     "km_gemm_fp8_rows_fused",
+    "km_gemm_fp8_blocks_fused",
     "km_gemm_fp8_tensor",
     "km_gemm_fp8_rows",
     "km_gemm_fp8_blocks",
@@ -76,6 +77,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.km_gemm_mx.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_gemm_mx_fused.argtypes = [p, i64, p, p, p, p, i64, i64, i64, i32, p]
     lib.km_gemm_fp8_rows_fused.argtypes = [p, i64, p, p, p, p, i64, i64, i64, i32, p]
+    lib.km_gemm_fp8_blocks_fused.argtypes = [p, i64, p, p, p, p, i64, i64, i64, i32, p]
     lib.km_gemm_fp8_tensor.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_gemm_fp8_rows.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_gemm_fp8_blocks.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
@@ -394,6 +396,32 @@ def gemm_fp8_rows_fused(x: Tensor, b: Tensor, b_scale: Tensor, bias: Tensor | No
     c = torch.empty(m, n, device=dev, dtype=x.dtype)
     with torch.cuda.device(dev):
         _check(load().km_gemm_fp8_rows_fused(x.data_ptr(), x.stride(0) if m else k, b.data_ptr(), b_scale.data_ptr(), None if bias is None else bias.data_ptr(), c.data_ptr(), m, n, k, _dtype_code(x.dtype), _stream(x)))
+    return c
+
+
+def gemm_fp8_blocks_fused(x: Tensor, b: Tensor, b_scale: Tensor, bias: Tensor | None) -> Tensor:
+    """The block-recipe linear in one launch: x `[M, K]` bf16 / fp16 is quantized per row and 128
+    columns inside the GEMM (same codes and scales as `quant_blocks(x, "act")`), b `[N, K]` e4m3,
+    b_scale `[ceil(N/128), K/128]` fp32; K % 128 == 0, N % 32 == 0. Meant for M up to `FUSED_MAX_M`."""
+    if x.dim() != 2 or b.dim() != 2 or x.shape[1] != b.shape[1]:
+        raise ValueError(f"operands must be [M, K] and [N, K], got {tuple(x.shape)} and {tuple(b.shape)}")
+    m, k = x.shape
+    n = b.shape[0]
+    if k % 128 or n % 32:
+        raise ValueError(f"the fused block linear needs K % 128 == 0 and N % 32 == 0, got K={k}, N={n}")
+    if b.dtype != E4M3 or tuple(b_scale.shape) != (-(-n // BLOCK), k // BLOCK) or b_scale.dtype != torch.float32:
+        raise ValueError(f"the weight must be float8_e4m3fn with fp32 block scales [{-(-n // BLOCK)}, {k // BLOCK}]")
+    dev = _on_gpu(x, b, b_scale, bias)
+    if x.stride(1) != 1 or x.stride(0) % 8 or x.stride(0) < k or x.data_ptr() % 16:
+        x = x.contiguous()
+    b, b_scale = b.contiguous(), b_scale.contiguous()
+    if bias is not None:
+        if bias.shape != (n,):
+            raise ValueError(f"bias must be [{n}], got {tuple(bias.shape)}")
+        bias = bias.to(x.dtype).contiguous()
+    c = torch.empty(m, n, device=dev, dtype=x.dtype)
+    with torch.cuda.device(dev):
+        _check(load().km_gemm_fp8_blocks_fused(x.data_ptr(), x.stride(0) if m else k, b.data_ptr(), b_scale.data_ptr(), None if bias is None else bias.data_ptr(), c.data_ptr(), m, n, k, _dtype_code(x.dtype), _stream(x)))
     return c
 
 

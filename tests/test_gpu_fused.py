@@ -115,7 +115,7 @@ def test_fused_mx_argument_errors_and_planner_candidate():
     assert not any(c["gemm"] == "fused" for c in fp8_linear.candidates("mx", 16, 48, 256))
     assert fp8_linear.candidates("row", 16, 256, 256)[-1]["gemm"] == "fused"
     assert not any(c["gemm"] == "fused" for c in fp8_linear.candidates("row", 32, 256, 256))
-    assert not any(c["gemm"] == "fused" for c in fp8_linear.candidates("block", 16, 256, 256))
+    assert fp8_linear.candidates("block", 16, 256, 256)[0]["gemm"] == "fused"
     assert not any(c["gemm"] == "fused" for c in fp8_linear.candidates("tensor", 16, 256, 256))
 
 
@@ -186,12 +186,60 @@ def test_fused_row_nonfinite_rows_follow_the_quantizer():
     assert rel_l2(fused[keep].double().cpu(), two[keep].double().cpu()) <= 4e-3
 
 
+# ---- block recipe ------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+@pytest.mark.parametrize("m,n,k", [(1, 32, 128), (5, 96, 384), (16, 256, 1024), (17, 64, 640), (32, 192, 384), (20, 160, 256), (33, 128, 512), (48, 192, 640), (64, 256, 3072), (100, 96, 896)])
+def test_fused_block_against_fp64_and_the_two_launch_path(dtype, m, n, k):
+    x, w, bias = operands(m, n, k, dtype, seed=m + n + 2)
+    w[: n // 2, : k // 2] *= 16.0   # weight blocks with different scales
+    xq, xs = formats.quantize(x, "block", "act")
+    wq, ws = formats.quantize(w, "block", "weight")
+    truth = linear.exact64(xq, xs, "block") @ linear.exact64(wq, ws, "block").T + bias.double()
+    eager = linear.fp8_forward(x, wq, ws, None, bias, "block")
+    y = native.gemm_fp8_blocks_fused(x.cuda(), wq.cuda(), ws.cuda(), bias.cuda())
+    assert y.shape == (m, n) and y.dtype == dtype
+    assert_no_regression(y.cpu(), eager, truth, f"fused block {m}x{n}x{k}")
+    assert rel_l2(y.cpu(), truth) <= REL_L2[dtype]
+    gq, gs = native.quant_blocks(x.cuda(), "act")
+    two = native.gemm_fp8_blocks(gq, gs, wq.cuda(), ws.cuda(), bias.cuda(), dtype, 1)
+    assert rel_l2(y.cpu(), two.double().cpu()) <= 2 * REL_L2[dtype]
+    y0 = native.gemm_fp8_blocks_fused(x.cuda(), wq.cuda(), ws.cuda(), None)
+    assert rel_l2(y0.cpu(), truth - bias.double()) <= REL_L2[dtype]
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+def test_fused_block_equals_the_two_launch_path_where_sums_are_exact(dtype):
+    """Every 128-column block of a row has the abs-max 7 * 2^e (scale 2^(e-6) exactly), x holds
+    small-integer multiples of 2^e and W small-integer codes with power-of-two block scales: all
+    partial sums are exact, so the one-launch kernel must give the bytes of quantizer + GEMM."""
+    for m, n, k in ((40, 96, 1024), (30, 128, 512)):
+        g = torch.Generator().manual_seed(7)
+        x = torch.randint(-6, 7, (m, k), generator=g).float()
+        for r in range(m):
+            for kb in range(k // 128):
+                e = (r + 2 * kb) % 3 - 1
+                x[r, kb * 128 : kb * 128 + 128] *= 2.0**e
+                x[r, kb * 128 + (r * 37 + kb) % 128] = 7 * 2.0**e
+        x[3] = 0
+        wq = torch.randint(-4, 5, (n, k), generator=g).float().to(torch.float8_e4m3fn)
+        ws = 2.0 ** torch.randint(-1, 2, (-(-n // 128), k // 128), generator=g).float()
+        # promoted terms are multiples of 1/4 below 2^14 and there are at most 8 of them: exact in fp32
+        xd = x.to(dtype).cuda()
+        assert torch.equal(xd.float().cpu(), x)
+        gq, gs = native.quant_blocks(xd, "act")
+        two = native.gemm_fp8_blocks(gq, gs, wq.cuda(), ws.cuda(), None, dtype, 1)
+        fused = native.gemm_fp8_blocks_fused(xd, wq.cuda(), ws.cuda(), None)
+        assert torch.equal(fused, two), (m, n, k)
+
+
 # ---- through the registered op ------------------------------------------------------------------
 
 
-@pytest.mark.parametrize("recipe", ("mx", "row"))
+@pytest.mark.parametrize("recipe", ("mx", "row", "block"))
 def test_short_m_through_the_registered_op(recipe, tmp_path, monkeypatch):
-    """`fp8_linear` at 8 rows: with timing off the planner binds its first candidate (mx: the
+    """`fp8_linear` at 8 rows: with timing off the planner binds its first candidate (mx and block: the
     one-launch kernel); with the table on it times the one-launch kernel among the tile
     configurations and stores a winner. Either way the result obeys the GEMM tolerance."""
     from kohakumosstrainer_amd.kernels import tuning
@@ -216,7 +264,7 @@ def test_short_m_through_the_registered_op(recipe, tmp_path, monkeypatch):
             assert rel_l2(y.cpu(), truth) <= REL_L2[torch.bfloat16], (recipe, mode)
             chosen = fp8_linear._select("fwd", x.cuda(), cw.q, cw.scale, cw.aux, bias.cuda(), recipe, False)
             if mode == "off":
-                assert chosen["gemm"] == ("fused" if recipe == "mx" else "hip")
+                assert chosen["gemm"] == ("hip" if recipe == "row" else "fused")
             else:
                 rows = list(tmp_path.rglob("fp8_fwd.json"))
                 assert len(rows) == 1 and "fused" in rows[0].read_text(), "the one-launch kernel was among the timed candidates"
