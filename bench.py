@@ -215,6 +215,28 @@ def other_configs(dev, reps):
         fused_call()
         two_calls()
         small[f"M{ms}"] = {"fused_us": event_ms(fused_call, reps) * 1e3, "quantizer_plus_gemm_us": event_ms(two_calls, reps) * 1e3}
+        # the block and row recipes at the same shape (weights quantized above: wbq / wbs, wq / ws)
+        st_ = torch.empty(k // 128, ms, dtype=torch.float32, device=dev)
+        sr_ = torch.empty(ms, dtype=torch.float32, device=dev)
+
+        def fused_block():
+            lib.km_gemm_fp8_blocks_fused(xs_.data_ptr(), k, wbq.data_ptr(), wbs.data_ptr(), None, y_.data_ptr(), ms, n, k, native.KM_BF16, stream)
+
+        def two_block():
+            lib.km_quant_blocks(xs_.data_ptr(), ms, k, k, 1, native.KM_BF16, native.ROLE_ACT, q_.data_ptr(), None, st_.data_ptr(), stream)
+            lib.km_gemm_fp8_blocks(q_.data_ptr(), st_.data_ptr(), wbq.data_ptr(), wbs.data_ptr(), None, y_.data_ptr(), ms, n, k, native.KM_BF16, native.SCALES_KMAJOR, 1, stream)
+
+        def fused_row():
+            lib.km_gemm_fp8_rows_fused(xs_.data_ptr(), k, wq.data_ptr(), ws.data_ptr(), None, y_.data_ptr(), ms, n, k, native.KM_BF16, stream)
+
+        def two_row():
+            lib.km_quant_rows(xs_.data_ptr(), ms, k, k, 1, native.KM_BF16, q_.data_ptr(), sr_.data_ptr(), stream)
+            lib.km_gemm_fp8_rows(q_.data_ptr(), sr_.data_ptr(), wq.data_ptr(), ws.data_ptr(), None, y_.data_ptr(), ms, n, k, native.KM_BF16, cfg_small, stream)
+
+        for fn in (fused_block, two_block, fused_row, two_row):
+            fn()
+        small[f"M{ms}"].update({"block_fused_us": event_ms(fused_block, reps) * 1e3, "block_quantizer_plus_gemm_us": event_ms(two_block, reps) * 1e3,
+                                "row_fused_us": event_ms(fused_row, reps) * 1e3, "row_quantizer_plus_gemm_us": event_ms(two_row, reps) * 1e3})
     out["mx_short_M_K3072_N9216"] = {**small, "weight_MB": n * k / 1e6, "note": "one launch (x quantized inside the GEMM) vs two; the weight streams once either way"}
     # int8 compute linear (per-row int8 activations, int8 MFMA GEMM, int32 accumulation), same shape
     w_scale = (w.float().abs().amax(1).clamp_min(1e-12) / 127.0)
