@@ -256,6 +256,12 @@ def quant_blocks(x: Tensor, role: str = "act", natural: bool = True, kmajor: boo
     if k % BLOCK:
         raise ValueError(f"fp8 block: K={k} is not a multiple of {BLOCK}")
     _on_gpu(x)
+    if role == "weight" and rows % BLOCK == 0 and rows > 1 and x.stride(0) == 1 and x.stride(1) >= rows:
+        # A transposed view (the W^T copy of the input gradient): its 128 x 128 blocks are the
+        # transposed blocks of the memory-order matrix, so codes and scales are the transposes of
+        # that matrix's, which the vector kernel quantizes at full bandwidth.
+        q, s = quant_blocks(x.t(), "weight")
+        return q.view(torch.uint8).t().contiguous().view(E4M3), s.t().contiguous()
     q = torch.empty(rows, k, device=x.device, dtype=torch.uint8)
     srows = rows if role == "act" else -(-rows // BLOCK)
     s = torch.empty(srows, k // BLOCK, device=x.device, dtype=torch.float32) if natural else None

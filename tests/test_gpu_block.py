@@ -64,10 +64,12 @@ def test_block_quantizer_bytes_equal_oracle(dtype, role, m, k):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("role", ("act", "weight"))
-@pytest.mark.parametrize("n,k", [(256, 384), (384, 128), (200, 256)])
+@pytest.mark.parametrize("n,k", [(256, 384), (384, 128), (200, 256), (256, 200), (128, 72)])
 def test_block_quantizer_transposed_view(dtype, role, n, k):
     """`quantize(w.t(), "block", role)` of the input-gradient weight copy: the operand is [K, N]
-    with unit stride down its rows; N must be a multiple of 128 only as its column count."""
+    with unit stride down its rows; N must be a multiple of 128 only as its column count. A weight
+    whose K is a multiple of 128 too is quantized in memory order and transposed; any other
+    (K = 200, 72) takes the element-wise kernel."""
     w = operand(n, k, dtype, seed=5)
     if n % 128:
         with pytest.raises(ValueError):
