@@ -65,7 +65,7 @@ def check(got, eager, exact, dtype, what, slack=1.0):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("recipe,dgrad", [("mx", True), ("mx", False), ("tensor", True), ("row", True), ("row", False)])
+@pytest.mark.parametrize("recipe,dgrad", [("mx", True), ("mx", False), ("tensor", True), ("row", True), ("row", False), ("block", True), ("block", False)])
 def test_fp8_linear_forward_and_grads(dtype, recipe, dgrad):
     m, n, k = 300, 384, 512
     x, w, bias, dy, base = problem(m, n, k, dtype, recipe, dgrad)
@@ -210,6 +210,31 @@ def test_trainable_fp8_cache_refreshes_from_the_device_quantizers():
     assert oracle_stats.rel_l2(lin.weight.grad.cpu(), ref_w) < 5e-3
     assert torch.equal(lin.bias.grad.cpu(), oracle_linear.bias_grad(g.cpu(), torch.bfloat16))
     exact_dx = exact_product(g.cpu(), tq, ts, None, "mx")
+    assert oracle_stats.rel_l2(x.grad.cpu(), exact_dx) < 2e-3
+
+
+def test_trainable_fp8_cache_block_recipe():
+    """The trainable-weight op under the block recipe: both copies come from the device block
+    quantizer (the W^T copy through the transposed view) and equal the host's bytes."""
+    torch.manual_seed(2)
+    lin = MossLinear(512, 384, bias=True).to(DEV, torch.bfloat16)
+    lin.init_weights(0.05)
+    attach_compute(nn.ModuleDict({"l": lin}), "fp8_compute", default_filter(()), torch.bfloat16, recipe="block", dgrad=True)
+    cache = lin.compute
+    assert cache.recipe == "block"
+    hq, hs = oracle_formats.quantize(lin.weight.detach().cpu(), "block", "weight")
+    assert torch.equal(cache.q.cpu().view(torch.uint8), hq.view(torch.uint8)) and torch.equal(cache.scale.cpu(), hs)
+    tq, ts = oracle_formats.quantize(lin.weight.detach().cpu().t().contiguous(), "block", "weight")
+    assert torch.equal(cache.q_t.cpu().view(torch.uint8), tq.view(torch.uint8)) and torch.equal(cache.scale_t.cpu(), ts)
+    x = torch.randn(256, 512, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    g = torch.randn(256, 384, device=DEV, dtype=torch.bfloat16)
+    y = lin(x)
+    y.backward(g)
+    exact_y = exact_product(x.detach().cpu(), hq, hs, lin.bias.detach().cpu(), "block")
+    assert oracle_stats.rel_l2(y.detach().cpu(), exact_y) < 2e-3
+    ref_w = (g.double().t() @ x.detach().double()).cpu()
+    assert oracle_stats.rel_l2(lin.weight.grad.cpu(), ref_w) < 5e-3
+    exact_dx = exact_product(g.cpu(), tq, ts, None, "block")
     assert oracle_stats.rel_l2(x.grad.cpu(), exact_dx) < 2e-3
 
 
