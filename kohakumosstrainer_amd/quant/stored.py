@@ -10,6 +10,8 @@ helpers `save_quantized` / `load_quantized` over safetensors.
 """
 
 import json
+import struct
+from dataclasses import dataclass
 from pathlib import Path
 
 import torch
@@ -23,53 +25,88 @@ SCALE = ".weight_scale"
 KEEP_FP32 = ("rope.bands",)
 
 
+@dataclass(frozen=True)
+class StoredRecord:
+    """What the `kohakumoss_fp8` metadata entry says: one recipe, the module paths stored as codes."""
+
+    recipe: str
+    layers: tuple[str, ...]
+
+    @classmethod
+    def parse(cls, raw: dict) -> "StoredRecord":
+        return cls(str(raw["recipe"]), tuple(raw["layers"]))
+
+    def as_dict(self) -> dict:
+        return {"recipe": self.recipe, "layers": list(self.layers)}
+
+    def metadata(self) -> dict[str, str]:
+        return {FP8_KEY: json.dumps(self.as_dict())}
+
+    @property
+    def weight_keys(self) -> set[str]:
+        return {path + ".weight" for path in self.layers}
+
+    @property
+    def scale_keys(self) -> set[str]:
+        return {path + SCALE for path in self.layers}
+
+
 def compute_bases(model: nn.Module) -> dict[str, ComputeWeight]:
     """{module path: ComputeWeight} of every fp8-compute MossLinear of `model`."""
-    return {path: lin.base for path, lin in model.named_modules() if isinstance(lin, MossLinear) and isinstance(lin.base, ComputeWeight)}
+    found = {}
+    for path, module in model.named_modules():
+        if isinstance(module, MossLinear) and isinstance(module.base, ComputeWeight):
+            found[path] = module.base
+    return found
+
+
+def _host(t: Tensor) -> Tensor:
+    return t.detach().contiguous().cpu()
 
 
 def quantized_state(model: nn.Module, keys: list[str], dtype: torch.dtype) -> tuple[dict[str, Tensor], dict[str, str]]:
-    """`(state, metadata)` of `model` over its state `keys`, on the host: fp8-compute layers as
-    codes and scale, every other floating-point tensor cast to `dtype` (the KEEP_FP32 names
-    stay fp32). One recipe per checkpoint."""
+    """`(state, metadata)` of `model` over its state `keys`, on the host: an fp8-compute layer
+    contributes its codes under `<path>.weight` and its scale under `<path>.weight_scale`, every
+    other floating-point tensor is cast to `dtype` (the KEEP_FP32 names stay as they are). A
+    checkpoint holds one recipe; a model with folded scales has no fp8 bases to export."""
     if getattr(model, "fold_scales", None) is not None:
         raise ValueError("a folded (fp16-fix) model is exported without fp8 bases")
     bases = compute_bases(model)
-    recipes = {b.recipe for b in bases.values()}
+    recipes = sorted({base.recipe for base in bases.values()})
     if len(recipes) != 1:
-        raise ValueError(f"one fp8 recipe per checkpoint, found {sorted(recipes)}")
-    live = {**dict(model.named_buffers()), **dict(model.named_parameters())}
+        raise ValueError(f"one fp8 recipe per checkpoint, found {recipes}")
+    tensors = dict(model.named_buffers())
+    tensors.update(model.named_parameters())
     state: dict[str, Tensor] = {}
     for key in keys:
-        path = key[: -len(".weight")] if key.endswith(".weight") else None
-        if path in bases:
-            state[key] = bases[path].q.contiguous().cpu()
-            state[path + SCALE] = bases[path].scale.contiguous().cpu()
-            continue
-        t = live[key].detach()
-        if key not in KEEP_FP32 and t.is_floating_point():
-            t = t.to(dtype)
-        state[key] = t.contiguous().cpu()
-    record = {"recipe": recipes.pop(), "layers": sorted(bases)}
-    return state, {FP8_KEY: json.dumps(record)}
+        owner = key.removesuffix(".weight") if key.endswith(".weight") else None
+        base = bases.get(owner) if owner is not None else None
+        if base is not None:
+            state[key], state[owner + SCALE] = _host(base.q), _host(base.scale)
+        else:
+            value = tensors[key]
+            cast = value.is_floating_point() and key not in KEEP_FP32
+            state[key] = _host(value.to(dtype) if cast else value)
+    return state, StoredRecord(recipes[0], tuple(sorted(bases))).metadata()
 
 
 def read_safetensors_metadata(path: str | Path) -> dict[str, str]:
-    """The `__metadata__` string map of a safetensors file (empty when it has none); reads the
-    header only."""
+    """The `__metadata__` string map of a safetensors file (empty when it has none). Only the
+    header is read: an 8-byte little-endian length, then that many bytes of JSON."""
     with open(path, "rb") as f:
-        size = int.from_bytes(f.read(8), "little")
-        header = json.loads(f.read(size))
-    return dict(header.get("__metadata__") or {})
+        (length,) = struct.unpack("<Q", f.read(8))
+        header = json.loads(f.read(length))
+    meta = header.get("__metadata__")
+    return dict(meta) if meta else {}
 
 
 def read_meta_record(path: str | Path, key: str) -> dict | None:
-    """The JSON record under metadata `key` of a single safetensors file, if it carries one."""
-    path = Path(path)
-    if not path.is_file():
+    """The JSON record under metadata `key` of a single safetensors file, or None when the path
+    is not a file or the key is absent."""
+    if not Path(path).is_file():
         return None
-    meta = read_safetensors_metadata(path)
-    return json.loads(meta[key]) if key in meta else None
+    raw = read_safetensors_metadata(path).get(key)
+    return None if raw is None else json.loads(raw)
 
 
 def read_record(path: str | Path) -> dict | None:
@@ -79,30 +116,35 @@ def read_record(path: str | Path) -> dict | None:
 
 def stored_keys(record: dict) -> tuple[set[str], set[str]]:
     """(the `.weight` keys of stored layers, their scale keys)."""
-    layers = record["layers"]
-    return {f"{p}.weight" for p in layers}, {p + SCALE for p in layers}
+    parsed = StoredRecord.parse(record)
+    return parsed.weight_keys, parsed.scale_keys
+
+
+def _reader(view):
+    """`view` is anything that hands out tensors by key: a dict, an open safetensors file."""
+    return view.get if hasattr(view, "get") else view.get_tensor
 
 
 @torch.no_grad()
 def attach_stored(model: nn.Module, view, record: dict, device, dtype: torch.dtype) -> int:
-    """Attach a ComputeWeight read from `view` (anything with `.get(key) -> Tensor`: a dict, an
-    open safetensors file) to every recorded layer, drop the layer's dense parameter and bind the
-    base for `(device, dtype)`; returns how many layers were attached."""
-    recipe = record["recipe"]
-    get = view.get if hasattr(view, "get") else view.get_tensor
-    for path in record["layers"]:
-        lin = model.get_submodule(path)
-        if not isinstance(lin, MossLinear):
-            raise TypeError(f"{path} is {type(lin).__name__}, not a MossLinear")
-        q = get(f"{path}.weight").to(device)
-        scale = get(path + SCALE).to(device)
-        if tuple(q.shape) != (lin.out_features, lin.in_features):
-            raise ValueError(f"{path}: stored codes are {tuple(q.shape)}, the layer is {(lin.out_features, lin.in_features)}")
-        base = ComputeWeight.from_stored(recipe, q, scale)
-        lin.weight = nn.Parameter(torch.empty(0, dtype=dtype, device=device), requires_grad=False)
-        lin.set_base(base)
+    """Give every recorded layer a ComputeWeight built from the codes and scale in `view`, replace
+    its dense parameter by an empty placeholder and bind the base for `(device, dtype)`. No 16-bit
+    copy of a stored weight is made at any point. Returns the number of layers attached."""
+    parsed = StoredRecord.parse(record)
+    read = _reader(view)
+    for path in parsed.layers:
+        layer = model.get_submodule(path)
+        if not isinstance(layer, MossLinear):
+            raise TypeError(f"{path} is {type(layer).__name__}, not a MossLinear")
+        codes = read(path + ".weight").to(device)
+        want = (layer.out_features, layer.in_features)
+        if tuple(codes.shape) != want:
+            raise ValueError(f"{path}: stored codes are {tuple(codes.shape)}, the layer is {want}")
+        base = ComputeWeight.from_stored(parsed.recipe, codes, read(path + SCALE).to(device))
+        layer.weight = nn.Parameter(torch.empty(0, dtype=dtype, device=device), requires_grad=False)
+        layer.set_base(base)
         base.bind(dtype, device)
-    return len(record["layers"])
+    return len(parsed.layers)
 
 
 def save_quantized(model: nn.Module, path: str | Path, dtype: torch.dtype = torch.bfloat16) -> dict:
