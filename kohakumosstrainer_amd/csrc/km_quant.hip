@@ -542,11 +542,24 @@ __global__ __launch_bounds__(256) void quant_i8_rows(const uint16_t* __restrict_
   m = wave_max(m);
   const float s = i8_scale_of(m);
   if (lane == 0) scale[row] = s;
+  // Without column scales the inputs are 16-bit patterns below the row's amax: the quotient then
+  // comes from the rounded reciprocal and two fused corrections, as in the fp8 row quantizer (equal
+  // to the division wherever the rounded quotient is not zero; the GPU tests compare every (amax, x)
+  // pair with the dividing element-wise kernel). Column-scaled inputs are arbitrary fp32 values and a
+  // row with an infinite amax follows the division's special cases: both divide.
+  const bool fast = col_scale == nullptr && m < kInfBits;
+  const float rcp = __fdiv_rn(1.0f, s);
   auto codes = [&](const uint4& r, uint32_t c) __attribute__((always_inline)) {
     scaled8<DT>(r, col_scale, c, f);
-    const uint32_t lo = i8_code(f[0], s) | (i8_code(f[1], s) << 8) | (i8_code(f[2], s) << 16) | (i8_code(f[3], s) << 24);
-    const uint32_t hi = i8_code(f[4], s) | (i8_code(f[5], s) << 8) | (i8_code(f[6], s) << 16) | (i8_code(f[7], s) << 24);
-    return make_uint2(lo, hi);
+    uint32_t b[8];
+    if (fast) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) b[i] = (uint32_t)(int)__builtin_amdgcn_fmed3f(__builtin_rintf(quotient(f[i], s, rcp)), -127.0f, 127.0f) & 0xFFu;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) b[i] = i8_code(f[i], s);
+    }
+    return make_uint2(b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24), b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24));
   };
   if constexpr (HELD) {
 #pragma unroll

@@ -75,6 +75,29 @@ def test_quantizer_every_bf16_pattern_under_sampled_amax():
     check_rows(x)
 
 
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+def test_quantizer_vector_kernel_equals_the_dividing_kernel_on_every_pair(dtype):
+    """Without column scales the vectorized kernel forms x / s from a rounded reciprocal and two
+    fused corrections; the element-wise kernel (taken for a view that is not 16-byte aligned)
+    divides. Every (amax, x) pair of finite 16-bit patterns with |x| <= amax must give the same
+    byte and the same scale."""
+    inf16 = 0x7F80 if dtype == torch.bfloat16 else 0x7C00
+    pats = torch.arange(0x10000, dtype=torch.int32, device="cuda")
+    chunk = 2048
+    for a0 in range(0, inf16, chunk):
+        amax = torch.arange(a0, min(a0 + chunk, inf16), device="cuda", dtype=torch.int32)
+        keep = (pats & 0x7FFF)[None, :] <= amax[:, None]
+        v = torch.where(keep, pats[None, :], torch.zeros((), dtype=torch.int32, device="cuda"))
+        x = (v - (v >= 0x8000).to(torch.int32) * 0x10000).to(torch.int16).view(dtype)
+        wide = torch.zeros(x.shape[0], x.shape[1] + 8, dtype=dtype, device="cuda")
+        wide[:, 1:-7] = x
+        q_fast, s_fast = native.quant_rows_i8(x)
+        q_div, s_div = native.quant_rows_i8(wide[:, 1:-7])
+        assert torch.equal(s_fast.view(torch.int32), s_div.view(torch.int32))
+        assert torch.equal(q_fast, q_div), f"amax patterns {a0}..{a0 + chunk}"
+        del x, wide, v, keep, q_fast, q_div
+
+
 def test_quantizer_full_size():
     g = torch.Generator().manual_seed(0)
     x = torch.randn(16384, 3072, generator=g)
