@@ -8,13 +8,13 @@
 //
 // Shape of the kernel. At short M the job is to stream the weight once, so there is no LDS
 // staging and no barrier in the K loop: a workgroup owns 16*TM tokens x 32 (or 64) output columns and
-// its four wavefronts split K (wavefront w takes K steps w, w+4, ...), each loading its MFMA
+// its four (eight for a single row tile) wavefronts split K (wavefront w takes K steps w, w+4, ...), each loading its MFMA
 // fragments straight from global memory in the MFMA's own layout (lane l: row l%16, K bytes
 // [16g, 16g+16) and [64+16g, 64+16g+16) with g = l/16), one to three steps ahead in registers. N/32
 // workgroups (288 at N = 9216) keep every compute unit streaming. A 32-column block of x lies in
 // two lanes (g and g^1); they share their 16-bit abs-max with one cross-lane exchange, and a
 // second one hands each lane the exponent byte the MFMA expects from it (lane g supplies block g).
-// The four partial sums of a workgroup meet in LDS at the end.
+// The partial sums of a workgroup meet in LDS at the end.
 #include <stdio.h>
 
 #include "km_gemm_common.h"
@@ -48,13 +48,15 @@ __device__ __forceinline__ uint32_t nonfinite_fix(uint32_t codes, uint32_t h, in
 // s[m, kb] * wscales[n / 128, kb]; wscales is then the [ceil(N/128), K/128] weight block scale matrix.
 constexpr int kFusedMx = 0, kFusedRow = 1, kFusedBlock = 2;
 
-template <int DT, int OUT, int TM, int TN, int MODE>
-__global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __restrict__ X, int64_t ldx, const uint8_t* __restrict__ B,
+// WAVES wavefronts split K (4, or 8 for a single row tile: three K steps each at K = 3072, all of
+// them in flight at once).
+template <int DT, int OUT, int TM, int TN, int MODE, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemm_mx_fused_kernel(const uint16_t* __restrict__ X, int64_t ldx, const uint8_t* __restrict__ B,
                                                             const uint8_t* __restrict__ Bs, const float* __restrict__ wscales,
                                                             const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N, int K) {
   constexpr bool ROW = MODE == kFusedRow, BLOCK = MODE == kFusedBlock;
   constexpr int BN = 16 * TN;  // 32 output columns, or 64: half as many workgroups quantize x again
-  __shared__ float4 partial[4][TM * TN][64];
+  __shared__ float4 partial[WAVES][TM * TN][64];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, g = lane >> 4;
@@ -93,11 +95,11 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
   float s_row[TM], r_row[TM];
   bool finite_row[TM], nan_row[TM];
   if constexpr (ROW) {
-    __shared__ uint32_t row_amax[4][TM][16];
+    __shared__ uint32_t row_amax[WAVES][TM][16];
     uint32_t m16[TM];
 #pragma unroll
     for (int j = 0; j < TM; ++j) m16[j] = 0;
-    for (int ks = wave; ks < nk; ks += 4) {
+    for (int ks = wave; ks < nk; ks += WAVES) {
 #pragma unroll
       for (int j = 0; j < TM; ++j) {
         const int m = m0 + j * 16 + r16;
@@ -120,8 +122,9 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
-      const uint32_t m01 = max(row_amax[0][j][r16], row_amax[1][j][r16]), m23 = max(row_amax[2][j][r16], row_amax[3][j][r16]);
-      const uint32_t mm = max(m01, m23);
+      uint32_t mm = row_amax[0][j][r16];
+#pragma unroll
+      for (int w = 1; w < WAVES; ++w) mm = max(mm, row_amax[w][j][r16]);
       s_row[j] = scale_of_amax16<DT>(mm);
       r_row[j] = __fdiv_rn(1.0f, s_row[j]);
       finite_row[j] = mm < inf16<DT>();
@@ -213,22 +216,22 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
     }
   };
 
-  // K steps wave, wave + 4, ...: the slabs of the next DEPTH - 1 steps are in flight while this one
+  // K steps wave, wave + WAVES, ...: the slabs of the next DEPTH - 1 steps are in flight while this one
   // is multiplied (a ring of register slabs, walked by a loop unrolled over the ring)
   constexpr int DEPTH = TM == 1 ? 4 : 2;
   Slab ring[DEPTH];
 #pragma unroll
   for (int d = 0; d + 1 < DEPTH; ++d)
-    if (wave + 4 * d < nk) load(ring[d], wave + 4 * d);
+    if (wave + WAVES * d < nk) load(ring[d], wave + WAVES * d);
   int ks = wave;
   while (ks < nk) {
     static_for<DEPTH>([&](auto d_tag) __attribute__((always_inline)) {
       constexpr int d = decltype(d_tag)::value;
       if (ks < nk) {
-        const int ahead = ks + 4 * (DEPTH - 1);
+        const int ahead = ks + WAVES * (DEPTH - 1);
         if (ahead < nk) load(ring[(d + DEPTH - 1) % DEPTH], ahead);
         compute(ring[d]);
-        ks += 4;
+        ks += WAVES;
       }
     });
   }
@@ -238,16 +241,16 @@ __global__ __launch_bounds__(256) void gemm_mx_fused_kernel(const uint16_t* __re
 #pragma unroll
     for (int j = 0; j < TM; ++j) partial[wave][t * TM + j][lane] = make_float4(acc[t][j][0], acc[t][j][1], acc[t][j][2], acc[t][j][3]);
   __syncthreads();
-  // tile i of the TM * TN is summed and stored by wavefront i % 4: lane (r16, g) holds C[m][n .. n+3]
+  // tile i of the TM * TN is summed and stored by wavefront i % WAVES: lane (r16, g) holds C[m][n .. n+3]
 #pragma unroll
   for (int i = 0; i < TM * TN; ++i) {
-    if ((i & 3) != wave) continue;
+    if (i % WAVES != wave) continue;
     const int t = i / TM, j = i % TM;
     const int m = m0 + j * 16 + r16, n = n0 + t * 16 + 4 * g;
     if (m >= M) continue;
     float4 v = partial[0][i][lane];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) {
+    for (int w = 1; w < WAVES; ++w) {
       const float4 o = partial[w][i][lane];
       v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
     }
@@ -268,7 +271,8 @@ template <int DT, int TM, int TN, int MODE>
 static void launch_fused(const void* x, int64_t ldx, const void* b, const void* bs, const float* wscales, const void* bias, void* c,
                          int M, int N, int K, hipStream_t st) {
   const dim3 grid((unsigned)(N / (16 * TN)), (unsigned)((M + 16 * TM - 1) / (16 * TM)));
-  hipLaunchKernelGGL((gemm_mx_fused_kernel<DT, DT, TM, TN, MODE>), grid, dim3(256), 0, st, (const uint16_t*)x, ldx, (const uint8_t*)b,
+  constexpr int WAVES = TM == 1 ? 8 : 4;
+  hipLaunchKernelGGL((gemm_mx_fused_kernel<DT, DT, TM, TN, MODE, WAVES>), grid, dim3(64 * WAVES), 0, st, (const uint16_t*)x, ldx, (const uint8_t*)b,
                      (const uint8_t*)bs, wscales, (const uint16_t*)bias, (uint16_t*)c, M, N, K);
 }
 

@@ -47,9 +47,9 @@ def candidates(recipe: str, m: int, n: int | None = None, k: int | None = None) 
         ranked = sorted(fits, key=lambda c: c["bm"])
     if recipe in ("mx", "row", "block") and m <= native.FUSED_MAX_M and (n is None or n % 32 == 0) and (k is None or k % 128 == 0):
         # measured at K3072 N9216, one launch against quantizer + GEMM. mx: 9.1 against 19 us at M = 1,
-        # 11.0 against 21 at M = 16, 15.4 against 21 at M = 32 (even at 48); block: 11.9 against 21.5, 13.3
+        # 11.0 against 21 at M = 16, 15.4 against 21 at M = 32 (even at 48); block: 10.6 against 21.4, 12.2
         # against 22.7, 19.2 against 23.0: first pick up to 16 rows, a timed candidate up to 32. row (a
-        # second pass over x for the row maxima): 11.9 against 14.6 us at M = 1, even at M = 16: only
+        # second pass over x for the row maxima): 10.8 against 14.6 us at M = 1, even at M = 16: only
         # ever a timed candidate, up to 16 rows.
         fused = {"gemm": "fused", "id": -1, "bm": 16 * -(-max(m, 1) // 16), "bn": 64 if (n or 64) % 64 == 0 else 32}
         if recipe in ("mx", "block"):
