@@ -1,20 +1,28 @@
-// One-launch fp8 linears for short M on gfx950 (mx, per-row and block recipes): C = Q(x) B^T (+ bias) with x [M,K] bf16 / fp16
-// quantized to MXFP8 inside the K loop (E8M0 exponent per 32 columns, e4m3 codes: the same
-// arithmetic as the row-wise quantizer kernel, so the codes are the ones km_quant_mx writes) and
-// B [N,K] e4m3 with its MFMA-packed E8M0 scales.
-// Replaces the reference's Triton _fused_mx_kernel / fused_mx_mm
-// (src/kohakumoss_kernels/backends/triton/fp8/fused.py:98-120,182-194): at M <= 256 the
+// One-launch fp8 linears for short M on gfx950: C = Q(x) B^T (+ bias) with x [M,K] bf16 / fp16
+// quantized inside the K loop and B [N,K] e4m3 quantized beforehand, in three recipes:
+//
+//   mx     E8M0 exponent per 32 columns, e4m3 codes (the arithmetic of the row-wise MX quantizer
+//          kernel, so the codes are the ones km_quant_mx writes); B comes with its MFMA-packed
+//          E8M0 scales and the block-scaled MFMA applies both
+//   row    one fp32 scale per token row (a prologue scans the rows for their abs-max), unit MFMA
+//          scales, s[m] * wscale[n] on the sum at the end
+//   block  one fp32 scale per row and 128 columns: a K step is one block, its MFMA sum starts from
+//          zero and is promoted with s[m, kb] * wscale[n / 128, kb]
+//
+// Replaces the reference's Triton fused kernels (src/kohakumoss_kernels/backends/triton/fp8/fused.py:
+// _fused_mx_kernel :98-120, _fused_row_kernel :35-68, _fused_block_kernel :71-95): at M <= 256 the
 // reference's linear is bound by launches, not by the MMA, and one launch replaces two.
 //
 // Shape of the kernel. At short M the job is to stream the weight once, so there is no LDS
-// staging and no barrier in the K loop: a workgroup owns 16*TM tokens x 32 (or 64) output columns and
-// its four (eight for a single row tile) wavefronts split K (wavefront w takes K steps w, w+4, ...), each loading its MFMA
-// fragments straight from global memory in the MFMA's own layout (lane l: row l%16, K bytes
-// [16g, 16g+16) and [64+16g, 64+16g+16) with g = l/16), one to three steps ahead in registers. N/32
-// workgroups (288 at N = 9216) keep every compute unit streaming. A 32-column block of x lies in
-// two lanes (g and g^1); they share their 16-bit abs-max with one cross-lane exchange, and a
-// second one hands each lane the exponent byte the MFMA expects from it (lane g supplies block g).
-// The partial sums of a workgroup meet in LDS at the end.
+// staging and no barrier in the K loop: a workgroup owns 16*TM tokens x 64 output columns (32 when
+// N is not a multiple of 64) and its WAVES wavefronts split K (wavefront w takes K steps w,
+// w + WAVES, ...), each loading its MFMA fragments straight from global memory in the MFMA's own
+// layout (lane l: row l%16, K bytes [16g, 16g+16) and [64+16g, 64+16g+16) with g = l/16), one to
+// three steps ahead in registers. N/64 workgroups (144 at N = 9216) stream the weight; every one
+// of them quantizes its rows of x again, which is what bounds the useful M. For mx, a 32-column
+// block of x lies in two lanes (g and g^1): they share their 16-bit abs-max with one cross-lane
+// exchange, and a second one hands each lane the exponent byte the MFMA expects from it (lane g
+// supplies block g). The partial sums of a workgroup meet in LDS at the end.
 #include <stdio.h>
 
 #include "km_gemm_common.h"
@@ -38,14 +46,6 @@ __device__ __forceinline__ uint32_t nonfinite_fix(uint32_t codes, uint32_t h, in
   return codes;
 }
 
-// ROW: the per-row recipe instead of mx (reference _fused_row_kernel, fused.py:35-68): a prologue
-// takes each token row's abs-max over all of K (the wavefronts scan their own K steps, the maxima
-// meet in LDS), the loop quantizes with s[m] = max(amax, 1e-12) / 448 and the quotient of the row
-// quantizer kernel, the MFMAs run with unit scales and s[m] * wscale[n] multiplies the sum at the end.
-// MODE kFusedBlock: the block recipe (reference _fused_block_kernel, fused.py:71-95): every K step is
-// one 128-column block, so a row's abs-max over the step is its block's (the four lanes that share
-// the row exchange theirs), the step's MFMA sum starts from zero and is promoted with
-// s[m, kb] * wscales[n / 128, kb]; wscales is then the [ceil(N/128), K/128] weight block scale matrix.
 constexpr int kFusedMx = 0, kFusedRow = 1, kFusedBlock = 2;
 
 // WAVES wavefronts split K (4, or 8 for a single row tile: three K steps each at K = 3072, all of
