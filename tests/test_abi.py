@@ -28,7 +28,7 @@ def test_header_symbols_are_exported_and_bound():
 def test_abi_version_and_config_catalogue():
     lib = native.load()
     assert lib.km_abi_version() == 1
-    for kernel in (native.KERNEL_GEMM_MX, native.KERNEL_GEMM_FP8, native.KERNEL_WO_FWD, native.KERNEL_WO_DGRAD):
+    for kernel in (native.KERNEL_GEMM_MX, native.KERNEL_GEMM_FP8, native.KERNEL_WO_FWD, native.KERNEL_WO_DGRAD, native.KERNEL_GEMM_BLOCKS):
         cfgs = native.configs(kernel)
         assert cfgs and all({"id", "bm", "bn", "bk"} <= set(c) for c in cfgs)
         assert [c["id"] for c in cfgs] == list(range(len(cfgs)))
@@ -43,6 +43,22 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert b"multiple of 32" in lib.km_last_error()
     assert lib.km_gemm_mx(None, None, None, None, None, None, 64, 64, 96, native.KM_BF16, 0, 0, None) < 0
     assert b"multiple of 128" in lib.km_last_error()
+    assert lib.km_quant_blocks(None, 4, 200, 200, 1, native.KM_BF16, native.ROLE_ACT, None, None, None, None) < 0
+    assert b"multiple of 128" in lib.km_last_error()
+    assert lib.km_quant_blocks(None, 4, 256, 256, 1, native.KM_BF16, 7, None, None, None, None) < 0
+    assert b"role" in lib.km_last_error()
+    assert lib.km_gemm_fp8_blocks(None, None, None, None, None, None, 64, 64, 256, native.KM_BF16, 5, 0, None) < 0
+    assert b"scale layout" in lib.km_last_error()
+    assert lib.km_gemm_fp8_blocks(None, None, None, None, None, None, 64, 64, 256, native.KM_BF16, native.SCALES_KMAJOR, 9, None) < 0
+    assert b"config" in lib.km_last_error()
+    for fused in (lib.km_gemm_mx_fused, lib.km_gemm_fp8_rows_fused, lib.km_gemm_fp8_blocks_fused):
+        assert fused(None, 256, None, None, None, None, 8, 48, 256, native.KM_BF16, None) < 0
+        assert b"multiple of 32" in lib.km_last_error()
+        assert fused(None, 200, None, None, None, None, 8, 64, 200, native.KM_BF16, None) < 0
+        assert b"multiple of 128" in lib.km_last_error()
+        assert fused(None, 256, None, None, None, None, 8, 64, 256, native.KM_BF16, None) < 0
+        assert b"null pointer" in lib.km_last_error()
+        assert fused(None, 256, None, None, None, None, 0, 64, 256, native.KM_BF16, None) == 0
     assert lib.km_scales_packed_bytes(16384, 3072) == 16384 * 96
     assert lib.km_scales_packed_bytes(100, 256) == 2 * 1 * 512
     assert lib.km_scales_packed_bytes(100, 96) == -1
