@@ -215,6 +215,8 @@ def other_configs(dev, reps):
         fused_call()
         two_calls()
         small[f"M{ms}"] = {"fused_us": event_ms(fused_call, reps) * 1e3, "quantizer_plus_gemm_us": event_ms(two_calls, reps) * 1e3}
+        # the bound at short M is the weight stream (codes + E8M0 scales read once)
+        small[f"M{ms}"]["fused_weight_stream_GBps"] = (n * k + n * k // 32) / small[f"M{ms}"]["fused_us"] / 1e3
         # the block and row recipes at the same shape (weights quantized above: wbq / wbs, wq / ws)
         st_ = torch.empty(k // 128, ms, dtype=torch.float32, device=dev)
         sr_ = torch.empty(ms, dtype=torch.float32, device=dev)
@@ -237,7 +239,7 @@ def other_configs(dev, reps):
             fn()
         small[f"M{ms}"].update({"block_fused_us": event_ms(fused_block, reps) * 1e3, "block_quantizer_plus_gemm_us": event_ms(two_block, reps) * 1e3,
                                 "row_fused_us": event_ms(fused_row, reps) * 1e3, "row_quantizer_plus_gemm_us": event_ms(two_row, reps) * 1e3})
-    out["mx_short_M_K3072_N9216"] = {**small, "weight_MB": n * k / 1e6, "note": "one launch (x quantized inside the GEMM) vs two; the weight streams once either way"}
+    out["mx_short_M_K3072_N9216"] = {**small, "weight_MB": n * k / 1e6, "hbm_peak_GBps": HBM_PEAK_GBS, "note": "one launch (x quantized inside the GEMM) vs two; the weight streams once either way"}
     # int8 compute linear (per-row int8 activations, int8 MFMA GEMM, int32 accumulation), same shape
     w_scale = (w.float().abs().amax(1).clamp_min(1e-12) / 127.0)
     w8 = torch.round(w.float() / w_scale[:, None]).clamp_(-127, 127).to(torch.int8)
