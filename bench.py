@@ -101,11 +101,16 @@ def other_configs(dev, reps):
     for name, (m, k, n), fmt in (("wo_int8_M4096_K3072_N3072", (4096, 3072, 3072), "int8"), ("wo_e4m3_M8192_K3072_N12288", (8192, 3072, 12288), "fp8")):
         x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(dev)
         if fmt == "int8":
+            # frozen int8 base: codes uniform in [-127, 127], scale |N(0,0.02)|/127 + 1e-6 per output row
             q = torch.randint(-127, 128, (n, k), generator=g).to(torch.int8).to(dev)
+            scale = (torch.randn(n, generator=g).abs() * 0.02 / 127 + 1e-6).to(dev)
         else:
-            q = (torch.randn(n, k, generator=g) * 100).to(torch.float8_e4m3fn).to(dev)
-        scale = (torch.rand(n, generator=g) * 1e-3 + 1e-6).to(dev)
-        bias = torch.zeros(n, dtype=torch.bfloat16, device=dev)
+            # per-tensor e4m3 base: W ~N(0,0.02) in bf16, one scale amax/448 broadcast to the rows
+            w16 = (torch.randn(n, k, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+            q, s1 = native.quant_tensor(w16)
+            scale = s1.reshape(1).expand(n).contiguous()
+            del w16
+        bias = (torch.randn(n, generator=g) * 0.01).to(torch.bfloat16).to(dev)
         dy = torch.randn(m, n, generator=g).to(torch.bfloat16).to(dev)
         native.wo_gemm_fwd(x, q, scale, bias, 0)
         native.wo_gemm_dgrad(dy, q, scale, 0)

@@ -90,7 +90,8 @@ constexpr int wait_vm_lgkm0(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070
 // one of them (a "memory" clobber keeps LDS reads from moving across). The hazard recognizer
 // does not look into inline asm either: an SGPR written by a VALU instruction (v_readfirstlane,
 // the reload of a spilled SGPR) must not be read by a vector-memory instruction within 5 wait
-// states, and m0 not within 1, hence the s_nop in front of each.
+// states, and m0 not within 1, hence the s_nop in front of each. The direct-to-LDS load takes its
+// LDS address from m0, which the statement writes itself and declares as clobbered.
 __device__ __forceinline__ uint32_t lds_offset(const void* p) {
   return (uint32_t)reinterpret_cast<uintptr_t>((lds_ptr_t)const_cast<void*>(p));
 }
@@ -103,7 +104,7 @@ __device__ __forceinline__ v4i raw_rsrc(const void* base, uint32_t bytes) {
 // each lane fetches 16 bytes at voffset (+ soffset); they land at lds_addr + 16 * lane
 __device__ __forceinline__ void hidden_dma_b128(const v4i& rsrc, uint32_t lds_addr, int voffset, int soffset) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               ::"s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+               ::"s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
 }
 __device__ __forceinline__ uint64_t hidden_load_b64(const v4i& rsrc, int voffset, int soffset) {
   uint64_t v;

@@ -111,6 +111,45 @@ def test_int8_weight_only_frozen_base_shape():
     assert torch.equal(native.wo_gemm_fwd(xg[perm].contiguous(), qg, sg, bg, 0), y[perm])
 
 
+def test_fp8_weight_only_per_tensor_scale_mlp_up_projection():
+    """The DiT MLP up-projection shape: x bf16 [8192, 3072] ~N(0,1) (eight packed samples; only
+    the token count matters to the linear), W bf16 ~N(0,0.02) [12288, 3072] quantized with ONE
+    scale s = amax / 448 (tensor / tensor division) and handed to the op as that value broadcast
+    to the 12288 rows, bf16 bias. Forward and input gradient: a 256-row slice against the fp64
+    product with the exactly dequantized weight next to the oracle's eager result (10x rule,
+    rel-L2 <= 2e-3 forward, 4e-3 for the gradient whose scale lies on the contraction axis), and
+    the whole output against row-permutation equivariance."""
+    from oracle import formats
+
+    m, k, n = 8192, 3072, 12288
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    g.manual_seed(1)
+    w = (torch.randn(n, k, generator=g) * 0.02).to(torch.bfloat16)
+    bias = (torch.randn(n, generator=g) * 0.01).to(torch.bfloat16)
+    g.manual_seed(2)
+    dy = (torch.randn(m, n, generator=g) * 0.01).to(torch.bfloat16)
+    q, s = formats.quantize(w, "tensor", "weight")
+    assert s.numel() == 1 and s.item() == (w.float().abs().amax() / torch.tensor(448.0)).item()
+    scale = s.reshape(1).expand(n).contiguous()
+    xg, qg, sg, bg, dyg = x.cuda(), q.cuda(), scale.cuda(), bias.cuda(), dy.cuda()
+    w64 = linear.wo_exact64(q, scale)
+    rows = torch.arange(3000, 3256)
+    perm = torch.randperm(m, generator=g).cuda()
+
+    y = native.wo_gemm_fwd(xg, qg, sg, bg, 0)
+    truth = x[rows].double() @ w64.T + bias.double()
+    assert_no_regression(y[rows].cpu(), linear.wo_forward(x[rows], q, scale, bias), truth, "e4m3 per-tensor fwd")
+    assert rel_l2(y[rows].cpu(), truth) <= 2e-3
+    assert torch.equal(native.wo_gemm_fwd(xg[perm].contiguous(), qg, sg, bg, 0), y[perm])
+
+    dx = native.wo_gemm_dgrad(dyg, qg, sg, 0)
+    truth_dx = dy[rows].double() @ w64
+    assert_no_regression(dx[rows].cpu(), linear.wo_dgrad(dy[rows], q, scale), truth_dx, "e4m3 per-tensor dgrad")
+    assert rel_l2(dx[rows].cpu(), truth_dx) <= 4e-3
+    assert torch.equal(native.wo_gemm_dgrad(dyg[perm].contiguous(), qg, sg, 0), dx[perm])
+
+
 def test_argument_errors():
     x = torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda")
     q = torch.zeros(16, 64, dtype=torch.int8, device="cuda")
