@@ -277,6 +277,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=200, help="untimed steps first (about 0.1 s: the card needs that long to reach its sustained clocks)")
     ap.add_argument("--config", type=int, default=-1, help="GEMM tile configuration; -1 times every configuration once, as the tuning table does, and takes the fastest")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--headline-only", action="store_true", help="only the headline step and its GEMM (for short profiler runs): no quantizer sweep, no other shapes, no CPU leg")
     ap.add_argument("--calibrate", action="store_true", help="also run 5 plain device copies of the activation tensor (a kernel of known HBM traffic, to scale profiler byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -330,6 +331,10 @@ def main():
         after.record()
     torch.cuda.synchronize()
     gemm_ms = sum(b.elapsed_time(a) for b, a in marks) / len(marks)
+    if args.headline_only:
+        achieved = GEMM_FLOP / (gemm_ms * 1e-3) / 1e12
+        print(json.dumps({"ms_per_step": ms_per_step, "gemm_ms": gemm_ms, "gemm_TFLOPs": achieved, "frac": achieved / FP8_PEAK_TFLOPS, "gemm_tile_config": config, "gemm_tile_configs_ms": tried}))
+        return
     rows_ms = event_ms(lambda: native.quant_mx(x), max(args.steps, 10))
     fused_rows_ms = event_ms(lambda: native.quant_mx(x, natural=False, packed=True), max(args.steps, 10))
     xt = x.t()
