@@ -184,6 +184,18 @@ int km_wo_gemm_dgrad(const void *dy, const void *q, const float *scale, void *dx
                      void *q_t_workspace, int64_t M, int64_t N, int64_t K, int q_format, int dtype,
                      int config, void *stream);
 
+/* km_wo_gemm_dgrad without a workspace argument and without any allocation: the transposed codes
+ * go to a static device array of KM_WO_DGRAD_STATIC_MAX_CODES bytes that the library holds on every
+ * GPU it runs on until the process ends. N*K beyond that is rejected (KM_ERR_UNSUPPORTED). Same
+ * result as km_wo_gemm_dgrad, bit for bit. All calls on one GPU share the array: calls that overlap
+ * on one GPU (two streams, two threads) race; calls on one stream are ordered and safe.
+ * No counterpart in the reference: it is for callers that cannot allocate device memory around
+ * the call (code under HIP graph capture, tight serving loops, harnesses that forbid it). */
+#define KM_WO_DGRAD_STATIC_MAX_CODES (64ll << 20)
+int km_wo_gemm_dgrad_static(const void *dy, const void *q, const float *scale, void *dx,
+                            int64_t M, int64_t N, int64_t K, int q_format, int dtype, int config,
+                            void *stream);
+
 /* Group Hadamard rotation (ConvRot): y[r, :] = x[r, :] . blockdiag(H_group), H_group the normalised
  * Kronecker power of H4 = [[1,1,1,-1],[1,1,-1,1],[1,-1,1,1],[-1,1,1,1]] (symmetric, its own
  * inverse), group in {4, 16, 64, 256, 1024} dividing cols; x and y [rows, cols] contiguous,

@@ -22,6 +22,8 @@
 #include <hip/hip_fp16.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "km_gemm_common.h"
 
 namespace km {
@@ -331,6 +333,37 @@ static int check_wo_args(const char* who, const void* a, const void* q, const fl
   return km_fail(KM_ERR_ARG, msg);
 }
 
+// ---- the entry point that allocates nothing ----------------------------------------------------
+// km_wo_gemm_dgrad_static keeps the transposed codes in this array instead of a caller's workspace.
+// Every GPU the library runs on holds its own copy at its own address for the life of the process;
+// host code never uses the array's name as an address, only the per-device pointer below.
+constexpr int64_t kStaticCodeBytes = KM_WO_DGRAD_STATIC_MAX_CODES;
+static __device__ __align__(256) uint8_t scratch[kStaticCodeBytes];
+constexpr int kMaxDevices = 64;
+static void* g_scratch_of_device[kMaxDevices];
+static std::mutex g_scratch_lock;
+
+// device address of `scratch` on the current device (looked up once per device)
+static int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return km_fail(KM_ERR_LAUNCH, "km_wo_gemm_dgrad_static: hipGetDevice failed");
+  if (dev < 0 || dev >= kMaxDevices) return km_fail(KM_ERR_UNSUPPORTED, "km_wo_gemm_dgrad_static: device index beyond 63");
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (!g_scratch_of_device[dev]) {
+    void* ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || !ptr) {
+      static thread_local char msg[160];
+      snprintf(msg, sizeof msg, "km_wo_gemm_dgrad_static: hipGetSymbolAddress: %s", hipGetErrorString(err));
+      return km_fail(KM_ERR_LAUNCH, msg);
+    }
+    g_scratch_of_device[dev] = ptr;
+  }
+  *out = g_scratch_of_device[dev];
+  return KM_OK;
+}
+
 }  // namespace km
 
 using namespace km;
@@ -356,4 +389,25 @@ extern "C" int km_wo_gemm_dgrad(const void* dy, const void* q, const float* scal
   }
   // dx[M, K] = dy[M, N] @ Wd[K, N]^T with Wd = round16(q_t * scale[contraction column])
   return dispatch_types<true>(dtype, q_format, config, dy, q_t_workspace, scale, nullptr, dx, (int)M, (int)K, (int)N, st);
+}
+
+extern "C" int km_wo_gemm_dgrad_static(const void* dy, const void* q, const float* scale, void* dx, int64_t M, int64_t N,
+                                       int64_t K, int q_format, int dtype, int config, void* stream) {
+  // the size limit first: it is a property of the call, whatever the pointers are
+  if (N > 0 && K > 0 && (N > kStaticCodeBytes || K > kStaticCodeBytes || N * K > kStaticCodeBytes)) {
+    static thread_local char msg[200];
+    snprintf(msg, sizeof msg, "km_wo_gemm_dgrad_static: N*K = %lld codes exceed the static workspace of %lld bytes; use km_wo_gemm_dgrad with a workspace",
+             (long long)(N * K), (long long)kStaticCodeBytes);
+    return km_fail(KM_ERR_UNSUPPORTED, msg);
+  }
+  int rc = check_wo_args("km_wo_gemm_dgrad_static", dy, q, scale, dx, M, N, K, q_format, dtype, config);
+  if (rc != KM_OK) return rc;
+  if (M == 0 || K == 0) return KM_OK;
+  void* codes_t = nullptr;
+  if (N > 0) {
+    rc = static_scratch(&codes_t);
+    if (rc != KM_OK) return rc;
+  }
+  // the transposition rewrites all N*K bytes the GEMM reads, so nothing of an earlier call shows
+  return km_wo_gemm_dgrad(dy, q, scale, dx, codes_t, M, N, K, q_format, dtype, config, stream);
 }

@@ -45,6 +45,7 @@ EXPORTS = (
     "km_gemm_i8_rows",
     "km_wo_gemm_fwd",
     "km_wo_gemm_dgrad",
+    "km_wo_gemm_dgrad_static",
     "km_group_hadamard",
     "km_num_configs",
     "km_config_desc",
@@ -84,6 +85,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.km_gemm_i8_rows.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_wo_gemm_fwd.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_wo_gemm_dgrad.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
+    lib.km_wo_gemm_dgrad_static.argtypes = [p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_group_hadamard.argtypes = [p, i64, i64, i32, i32, p, p]
     lib.km_num_configs.argtypes = [i32]
     lib.km_config_desc.argtypes = [i32, i32, c.c_char_p, i32]
@@ -535,6 +537,30 @@ def wo_gemm_dgrad(dy: Tensor, q: Tensor, scale: Tensor, config: int = 0) -> Tens
     with torch.cuda.device(dy.device):
         _check(load().km_wo_gemm_dgrad(dy.data_ptr(), q.data_ptr(), scale.data_ptr(), dx.data_ptr(), work.data_ptr(), m, n, k, _QFORMATS[q.dtype], _dtype_code(dy.dtype), config, _stream(dy)))
     return dx
+
+
+WO_DGRAD_STATIC_MAX_CODES = 64 << 20  # bytes of the library's static transpose workspace per GPU
+
+
+def wo_gemm_dgrad_static(dy: Tensor, q: Tensor, scale: Tensor, out: Tensor, config: int = 0) -> Tensor:
+    """`wo_gemm_dgrad` into the caller's `out` `[M, K]` through the entry point that allocates
+    nothing: the transposed codes live in a static device array of the library (N * K up to
+    `WO_DGRAD_STATIC_MAX_CODES`). Operands must already be contiguous (fp32 scale); calls that
+    overlap on one GPU share that array and race."""
+    if dy.dim() != 2 or q.dim() != 2 or dy.shape[1] != q.shape[0]:
+        raise ValueError(f"dy must be [M, N] and q [N, K], got {tuple(dy.shape)} and {tuple(q.shape)}")
+    m, n = dy.shape
+    k = q.shape[1]
+    if q.dtype not in _QFORMATS or scale.dtype != torch.float32 or tuple(scale.shape) != (n,):
+        raise ValueError("codes must be int8 / float8_e4m3fn with an fp32 scale per row")
+    if tuple(out.shape) != (m, k) or out.dtype != dy.dtype:
+        raise ValueError(f"out must be [{m}, {k}] {dy.dtype}")
+    if not all(t.is_contiguous() for t in (dy, q, scale, out)):
+        raise ValueError("the no-allocation entry point takes contiguous operands")
+    _on_gpu(dy, q, scale, out)
+    with torch.cuda.device(dy.device):
+        _check(load().km_wo_gemm_dgrad_static(dy.data_ptr(), q.data_ptr(), scale.data_ptr(), out.data_ptr(), m, n, k, _QFORMATS[q.dtype], _dtype_code(dy.dtype), config, _stream(dy)))
+    return out
 
 
 def configs(kernel: int) -> list[dict]:
