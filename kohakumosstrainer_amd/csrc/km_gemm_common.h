@@ -102,10 +102,20 @@ __device__ __forceinline__ v4i raw_rsrc(const void* base, uint32_t bytes) {
              __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
 }
 // each lane fetches 16 bytes at voffset (+ soffset); they land at lds_addr + 16 * lane
+// (the compiler keeps m0 out of its own allocation and says so when it sees it in a clobber list)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void hidden_dma_b128(const v4i& rsrc, uint32_t lds_addr, int voffset, int soffset) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                ::"s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
 }
+// 4 bytes per lane to lds_addr + 4 * lane: used to pull lines into L2 ahead of their real fetch,
+// aimed at LDS bytes that a later load of the same wavefront overwrites
+__device__ __forceinline__ void hidden_touch_b32(const v4i& rsrc, uint32_t lds_addr, int voffset, int soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dword %1, %2, %3 offen lds"
+               ::"s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
+}
+#pragma clang diagnostic pop
 __device__ __forceinline__ uint64_t hidden_load_b64(const v4i& rsrc, int voffset, int soffset) {
   uint64_t v;
   asm volatile("s_nop 4\n\tbuffer_load_dwordx2 %0, %1, %2, %3 offen" : "=v"(v) : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
@@ -153,7 +163,7 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
     // sub-tile through LDS (idle now), 64 rows at a time: 8-byte LDS writes in the MFMA
     // layout, 16-byte LDS reads along rows, 16-byte global stores that cover whole
     // WTN*2-byte row segments (full 128-byte lines).
-    constexpr int RP = WTN * 2 + 32;            // LDS row pitch in bytes (pad spreads banks)
+    constexpr int RP = WTN * 2 + 16;            // LDS row pitch in bytes: 16 lanes x 2 column groups of a write land in 64 different banks
     constexpr int kMinBuf = (BM < BN ? BM : BN) * 128;
     constexpr int HM0 = TM < 4 ? TM : 4;        // MFMA tiles (of 16 rows) per pass, halved until
     constexpr int HM = HM0 * 16 * RP <= kMinBuf ? HM0 : (HM0 / 2) * 16 * RP <= kMinBuf ? HM0 / 2 : 1;  // it fits a buffer

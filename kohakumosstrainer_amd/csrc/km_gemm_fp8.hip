@@ -93,7 +93,10 @@ __device__ __forceinline__ void mfma_i8_half(v4f& c, const v8i& a, const v8i& b)
 // each other's waits, prologue and epilogue.
 // I8: int8 codes on the int32 MFMA (no block scales), scale vectors applied in the reference's
 // order of roundings at the store.
-template <int BM, int BN, bool MX, bool SCALE_KM, int OUT, bool A1, bool I8>
+// B3: a third B buffer (the whole 160 KiB of LDS). Every fetch of a step (A, B, and the scale lines
+// as a touch that only fills L2) is issued two steps before its use instead of one for B and the
+// scales: a load that misses the XCD's L2 takes longer than one step to arrive.
+template <int BM, int BN, bool MX, bool SCALE_KM, int OUT, bool A1, bool I8, bool B3 = false>
 __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ As, const uint8_t* __restrict__ B,
     const uint8_t* __restrict__ Bs, const float* __restrict__ sa, const float* __restrict__ sb,
@@ -103,13 +106,18 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
   constexpr int TM = WTM / 16, TN = WTN / 16;
   constexpr int A_BYTES = BM * kStepBytes, B_BYTES = BN * kStepBytes;
   constexpr int A_LD = BM / 32, B_LD = BN / 32;  // 32 rows (4 KiB) per pass of 256 lanes
-  constexpr int kWaitAllButA = wait_vm_lgkm0(A1 ? 0 : A_LD);  // all but the A_LD newest loads done (A1: all)
+  static_assert(!(A1 && B3), "the third B buffer goes with two A buffers");
+  constexpr int kTouches = (B3 && MX && SCALE_KM) ? 2 : 0;
+  // loads of this step that may still be in flight at its end: A1 none, else the A passes (and, B3, the
+  // B passes and scale touches, all issued after the step's own scale fetch)
+  constexpr int kWaitAllButA = wait_vm_lgkm0(A1 ? 0 : B3 ? A_LD + B_LD + kTouches : A_LD);
   static_assert(BM % 32 == 0 && BN % 32 == 0 && TM >= 1 && TN >= 2, "tile");
   static_assert(TM * (TN - 1) >= BM / 32 + BN / 32, "every fetch pass needs its own MFMA slot");
   __shared__ __attribute__((aligned(1024))) uint8_t a_buf0[A_BYTES];
   __shared__ __attribute__((aligned(1024))) uint8_t a_buf1[A1 ? 16 : A_BYTES];
   __shared__ __attribute__((aligned(1024))) uint8_t b_buf0[B_BYTES];
   __shared__ __attribute__((aligned(1024))) uint8_t b_buf1[B_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t b_buf2[B3 ? B_BYTES : 16];
 
   int tile_m, tile_n;
   tile_of(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, tile_n);
@@ -183,23 +191,36 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
   uint64_t wraw64 = 0, xraw64 = 0;  // packed layout: the 8 scale bytes of a lane
 
   // one 4 KiB pass (32 rows) of a slab: each wavefront moves 1 KiB with one instruction
-  auto dma_a_pass = [&](uint8_t* buf, int koff, int i) __attribute__((always_inline)) {
-    hidden_dma_b128(a_rsrc, lds_offset(buf) + i * 4096 + wave * 1024, ld_voff + i * pass_stride, koff);
+  // LDS buffers are named by their LDS byte address (uniform 32-bit values): the B buffers of the
+  // three-buffer variant change roles from step to step
+  auto dma_a_pass = [&](uint32_t buf, int koff, int i) __attribute__((always_inline)) {
+    hidden_dma_b128(a_rsrc, buf + i * 4096 + wave * 1024, ld_voff + i * pass_stride, koff);
   };
   // `beyond` (0 or 2^31) pushes the per-lane offset past the descriptor's range: the pass then
   // fills its LDS rows with zeros
-  auto dma_b_pass = [&](uint8_t* buf, int koff, int i, int beyond = 0) __attribute__((always_inline)) {
-    hidden_dma_b128(b_rsrc, lds_offset(buf) + i * 4096 + wave * 1024, ld_voff + i * pass_stride + beyond, koff);
+  auto dma_b_pass = [&](uint32_t buf, int koff, int i, int beyond = 0) __attribute__((always_inline)) {
+    hidden_dma_b128(b_rsrc, buf + i * 4096 + wave * 1024, ld_voff + i * pass_stride + beyond, koff);
   };
-  auto dma_a = [&](uint8_t* buf, int ks) __attribute__((always_inline)) {
+  auto dma_a = [&](uint32_t buf, int ks) __attribute__((always_inline)) {
     const int koff = __builtin_amdgcn_readfirstlane(ks * kStepBytes);
 #pragma unroll
     for (int i = 0; i < A_LD; ++i) dma_a_pass(buf, koff, i);
   };
-  auto dma_b = [&](uint8_t* buf, int ks) __attribute__((always_inline)) {
+  auto dma_b = [&](uint32_t buf, int ks, int beyond = 0) __attribute__((always_inline)) {
     const int koff = __builtin_amdgcn_readfirstlane(ks * kStepBytes);
 #pragma unroll
-    for (int i = 0; i < B_LD; ++i) dma_b_pass(buf, koff, i);
+    for (int i = 0; i < B_LD; ++i) dma_b_pass(buf, koff, i, beyond);
+  };
+  // B3: the 2 x 512 scale bytes this wavefront will fetch for step ks, requested early so that the
+  // fetch finds them in L2; the 2 x 256 bytes land in the first bytes of `scratch`'s pass 0 slot of
+  // this wavefront, which its own B pass 0 (issued later, so arriving later) overwrites
+  auto scale_touch = [&](int ks, uint32_t scratch) __attribute__((always_inline)) {
+    if constexpr (kTouches > 0) {
+      const int wso = __builtin_amdgcn_readfirstlane(ks * ws_step + ws_base);
+      const int xso = __builtin_amdgcn_readfirstlane(ks * xs_step + xs_base);
+      hidden_touch_b32(ws_rsrc, scratch + wave * 1024, ws_off[0], wso);
+      hidden_touch_b32(xs_rsrc, scratch + wave * 1024 + 256, xs_off[0], xso);
+    }
   };
   auto scale_fetch = [&](int ks) __attribute__((always_inline)) {
     if constexpr (MX) {
@@ -239,9 +260,10 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
       for (int t = 0; t < TM; ++t) xscale[P][t] = (int)((xraw[t] >> (8 * g)) & live);
     }
   };
-  auto fragment = [&](const uint8_t* slab, int row) __attribute__((always_inline)) -> v8i {
-    const v4i lo = *reinterpret_cast<const v4i*>(slab + slab_offset(row, g));
-    const v4i hi = *reinterpret_cast<const v4i*>(slab + slab_offset(row, g + 4));
+  typedef __attribute__((address_space(3))) const v4i* lds_v4i_cptr;
+  auto fragment = [&](uint32_t slab, int row) __attribute__((always_inline)) -> v8i {
+    const v4i lo = *(lds_v4i_cptr)(slab + slab_offset(row, g));
+    const v4i hi = *(lds_v4i_cptr)(slab + slab_offset(row, g + 4));
     return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
   // One K step with parity P: A(k) is already in registers, B(k) is in b_cur. Fetches B(k+1)
@@ -256,16 +278,21 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
   // over the first third, A passes over the rest): a wavefront that queues them back to back
   // blocks on the address unit it shares with the other three and issues no MFMA meanwhile.
   constexpr int kWindow = TM * (TN - 1);           // MFMAs before the last group
-  constexpr int kBWindow = kWindow / 3 > B_LD ? kWindow / 3 : B_LD;
-  auto step = [&](uint8_t* a_cur, uint8_t* a_nxt, uint8_t* b_cur, uint8_t* b_nxt, int ks, auto set_tag)
+  // (B3: both are needed two steps on, so the window is shared in proportion)
+  constexpr int kBWindow = B3 ? kWindow * B_LD / (A_LD + B_LD) : kWindow / 3 > B_LD ? kWindow / 3 : B_LD;
+  // b_fill: the buffer this step's B passes write, B(k+1) into b_nxt without B3, B(k+2) into the
+  // third buffer with it (free since the barrier at the end of step k-1, whose b_cur it was)
+  constexpr int kBAhead = B3 ? 2 : 1;
+  auto step = [&](uint32_t a_cur, uint32_t a_nxt, uint32_t b_cur, uint32_t b_nxt, uint32_t b_fill, int ks, auto set_tag)
                   __attribute__((always_inline)) {
     constexpr int P = decltype(set_tag)::value;
     const int next = min(ks + 1, nk - 1);
-    const int koff_b = __builtin_amdgcn_readfirstlane(next * kStepBytes);
+    const int koff_b = __builtin_amdgcn_readfirstlane(min(ks + kBAhead, nk - 1) * kStepBytes);
     const int koff_a = __builtin_amdgcn_readfirstlane(min(ks + (A1 ? 1 : 2), nk - 1) * kStepBytes);
     // int8 has no scale to zero the padding step of an odd step count with: its B slab is zeros
-    const int b_beyond = I8 ? __builtin_amdgcn_readfirstlane(ks + 1 >= nk ? (int)0x80000000 : 0) : 0;
+    const int b_beyond = I8 ? __builtin_amdgcn_readfirstlane(ks + kBAhead >= nk ? (int)0x80000000 : 0) : 0;
     scale_fetch(next);
+    scale_touch(min(ks + 3, nk - 1), b_fill);
     __builtin_amdgcn_sched_barrier(0);
     static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
       constexpr int t = decltype(t_tag)::value;
@@ -304,7 +331,7 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
             constexpr int i = decltype(i_tag)::value;
             if constexpr (q == (A1 ? i : i * kBWindow / B_LD)) {
               __builtin_amdgcn_sched_barrier(0);
-              dma_b_pass(b_nxt, koff_b, i, b_beyond);
+              dma_b_pass(b_fill, koff_b, i, b_beyond);
               __builtin_amdgcn_sched_barrier(0);
             }
           });
@@ -341,24 +368,44 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
   using set0_t = std::integral_constant<int, 0>;
   using set1_t = std::integral_constant<int, 1>;
 
-  // prologue: A(0), B(0), A(1) and the scales of step 0
-  dma_a(a_buf0, 0);
-  dma_b(b_buf0, 0);
+  // prologue: A(0), B(0), A(1) (B3: and B(1)) and the scales of step 0
+  const uint32_t la0 = lds_offset(a_buf0), la1 = A1 ? la0 : lds_offset(a_buf1);
+  const uint32_t lb0 = lds_offset(b_buf0), lb1 = lds_offset(b_buf1), lb2 = lds_offset(b_buf2);
+  dma_a(la0, 0);
+  dma_b(lb0, 0);
   scale_fetch(0);
-  if constexpr (!A1) dma_a(a_buf1, min(1, nk - 1));
+  if constexpr (!A1) dma_a(la1, min(1, nk - 1));
+  if constexpr (B3) {
+    dma_b(lb1, min(1, nk - 1), I8 && nk < 2 ? (int)0x80000000 : 0);
+    scale_touch(min(1, nk - 1), lb2);
+    scale_touch(min(2, nk - 1), lb2);
+  }
   __builtin_amdgcn_s_waitcnt(kWaitVm0);
   __syncthreads();
   if constexpr (!I8) scale_commit(set0_t{}, 0xFFFFFFFFu);
 #pragma unroll
-  for (int j = 0; j < TM; ++j) xf[j] = fragment(a_buf0, wm + j * 16 + r16);
-  wcur = fragment(b_buf0, wn + r16);
+  for (int j = 0; j < TM; ++j) xf[j] = fragment(la0, wm + j * 16 + r16);
+  wcur = fragment(lb0, wn + r16);
 
   // two steps per trip, one per buffer parity; an odd step count is padded with a zero-scaled
   // step (int8: a step whose B slab is zeros)
   const int nsteps = (nk + 1) & ~1;
-  for (int ks = 0; ks < nsteps; ks += 2) {
-    step(a_buf0, A1 ? a_buf0 : a_buf1, b_buf0, b_buf1, ks, set0_t{});
-    step(A1 ? a_buf0 : a_buf1, a_buf0, b_buf1, b_buf0, ks + 1, set1_t{});
+  if constexpr (B3) {
+    // the three B buffers take the roles (multiplied now, next, being filled) in turn
+    uint32_t b_now = lb0, b_next = lb1, b_fill = lb2;
+    for (int ks = 0; ks < nsteps; ks += 2) {
+      step(la0, la1, b_now, b_next, b_fill, ks, set0_t{});
+      step(la1, la0, b_next, b_fill, b_now, ks + 1, set1_t{});
+      const uint32_t was_now = b_now;
+      b_now = b_fill;
+      b_fill = b_next;
+      b_next = was_now;
+    }
+  } else {
+    for (int ks = 0; ks < nsteps; ks += 2) {
+      step(la0, la1, lb0, lb1, lb1, ks, set0_t{});
+      step(la1, la0, lb1, lb0, lb0, ks + 1, set1_t{});
+    }
   }
   __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));  // the last (clamped) prefetches and fragment reads must be done before LDS is reused
 
@@ -389,25 +436,26 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
 }
 
 struct GemmConfig {
-  int bm, bn;
+  int bm, bn, b_stages;
 };
 // Largest tile first: the host-side table ranks candidates the way the reference ranks its
 // Triton tiles (large tiles for large M). Four wavefronts in a 2 x 2 grid each.
 static const GemmConfig kGemmConfigs[] = {
-    {256, 256},
-    {128, 256},
-    {256, 128},
-    {128, 128},
-    {64, 128},
+    {256, 256, 2},
+    {128, 256, 2},
+    {256, 128, 2},
+    {128, 128, 2},
+    {64, 128, 2},
+    {256, 256, 3},
 };
 constexpr int kNumGemmConfigs = sizeof(kGemmConfigs) / sizeof(kGemmConfigs[0]);
 
-template <int BM, int BN, bool MX, bool SCALE_KM, int OUT, bool A1, bool I8>
+template <int BM, int BN, bool MX, bool SCALE_KM, int OUT, bool A1, bool I8, bool B3 = false>
 static int launch_gemm(const void* a, const void* as, const void* b, const void* bs, const float* sa,
                        const float* sb, const void* bias, void* c, int M, int N, int K, int scale_vectors,
                        hipStream_t st) {
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  hipLaunchKernelGGL((gemm_fp8_kernel<BM, BN, MX, SCALE_KM, OUT, A1, I8>), dim3(tiles), dim3(256), 0, st,
+  hipLaunchKernelGGL((gemm_fp8_kernel<BM, BN, MX, SCALE_KM, OUT, A1, I8, B3>), dim3(tiles), dim3(256), 0, st,
                      (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b, (const uint8_t*)bs, sa, sb,
                      (const uint16_t*)bias, (uint16_t*)c, M, N, K, scale_vectors);
   return km_check_launch("km_gemm");
@@ -423,6 +471,7 @@ static int dispatch_config(int config, const void* a, const void* as, const void
     case 2: return launch_gemm<256, 128, MX, SCALE_KM, OUT, false, I8>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
     case 3: return launch_gemm<128, 128, MX, SCALE_KM, OUT, false, I8>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
     case 4: return launch_gemm<64, 128, MX, SCALE_KM, OUT, false, I8>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
+    case 5: return launch_gemm<256, 256, MX, SCALE_KM, OUT, false, I8, true>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
   }
   return km_fail(KM_ERR_ARG, "km_gemm: unknown config");
 }
@@ -461,7 +510,7 @@ int gemm_num_configs() { return kNumGemmConfigs; }
 int gemm_config_desc(int config, char* buf, int len) {
   if (config < 0 || config >= kNumGemmConfigs) return km_fail(KM_ERR_ARG, "config out of range");
   const GemmConfig& c = kGemmConfigs[config];
-  snprintf(buf, len, "bm=%d,bn=%d,bk=128,waves=4,wg_per_cu=%d", c.bm, c.bn, config == 1 || config >= 3 ? 2 : 1);
+  snprintf(buf, len, "bm=%d,bn=%d,bk=128,waves=4,wg_per_cu=%d,b_stages=%d", c.bm, c.bn, config == 1 || config == 3 || config == 4 ? 2 : 1, c.b_stages);
   return KM_OK;
 }
 
