@@ -19,10 +19,10 @@ import torch
 from kohakumosstrainer_amd import native
 from kohakumosstrainer_amd.kernels import registry, tuning
 from kohakumosstrainer_amd.kernels.constraints import requires
+from kohakumosstrainer_amd.kernels.hadamard import HALF
 from kohakumosstrainer_amd.kernels.errors import BackendUnavailable
 from kohakumosstrainer_amd.kernels.fp8.formats import dequantize, packed_numel
-from kohakumosstrainer_amd.kernels.fp8.op import make_fp8_linear, make_fp8_linear_infer, register_launchers
-from kohakumosstrainer_amd.kernels.fp8.train import make_fp8_linear_train
+from kohakumosstrainer_amd.kernels.fp8.op import OPS, register_launchers
 from kohakumosstrainer_amd.kernels.tuning import pow2
 
 GPU_RECIPES = ("mx", "tensor", "row", "block")
@@ -135,5 +135,5 @@ def _gpu_recipe(query):
 
 
 register_launchers("hip", fwd, dgrad)
-for _op, _make in (("fp8_linear", make_fp8_linear), ("fp8_linear_infer", make_fp8_linear_infer), ("fp8_linear_train", make_fp8_linear_train)):
-    registry.register(_op, "hip", _make("hip"), supports=requires(kinds=("hip",), archs=("gfx950",), extra=_gpu_recipe))
+for _op, _make in OPS.items():
+    registry.register(_op, "hip", _make("hip"), supports=requires(kinds=("hip",), archs=("gfx950",), dtypes=HALF, extra=_gpu_recipe))

@@ -10,6 +10,7 @@ made per call as the reference makes its column-major copy (`int8/formats.py:55-
 from kohakumosstrainer_amd import native
 from kohakumosstrainer_amd.kernels import registry, tuning
 from kohakumosstrainer_amd.kernels.constraints import requires
+from kohakumosstrainer_amd.kernels.hadamard import HALF
 from kohakumosstrainer_amd.kernels.hadamard import rotate_2d
 from kohakumosstrainer_amd.kernels.int8.op import int8_supported, make_int8_linear, register_launchers
 from kohakumosstrainer_amd.kernels.tuning import pow2
@@ -67,4 +68,4 @@ def dgrad(dy, q, scale, group, mode):
 
 
 register_launchers("hip", fwd, dgrad)
-registry.register("int8_linear", "hip", make_int8_linear("hip"), supports=requires(kinds=("hip",), archs=("gfx950",), extra=int8_supported))
+registry.register("int8_linear", "hip", make_int8_linear("hip"), supports=requires(kinds=("hip",), archs=("gfx950",), dtypes=HALF, extra=int8_supported))

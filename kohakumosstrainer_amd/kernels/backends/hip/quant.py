@@ -7,6 +7,7 @@ gradient dx = dy @ round16(q * scale). Host-side counterpart of reference
 from kohakumosstrainer_amd import native
 from kohakumosstrainer_amd.kernels import registry, tuning
 from kohakumosstrainer_amd.kernels.constraints import requires
+from kohakumosstrainer_amd.kernels.hadamard import HALF
 from kohakumosstrainer_amd.kernels.hadamard import rotate_2d
 from kohakumosstrainer_amd.kernels.quant import fmt_supported, make_quant_linear, register_launchers
 from kohakumosstrainer_amd.kernels.rotated import compose, group_supported, make_quant_linear_rotated, register_rotated_launchers
@@ -54,7 +55,7 @@ def _format_supported(query):
 
 
 register_launchers("hip", fwd, dgrad)
-registry.register("quant_linear", "hip", make_quant_linear("hip"), supports=requires(kinds=("hip",), archs=("gfx950",), extra=_format_supported))
+registry.register("quant_linear", "hip", make_quant_linear("hip"), supports=requires(kinds=("hip",), archs=("gfx950",), dtypes=HALF, extra=_format_supported))
 
 
 def _rotated_supported(query):
@@ -64,4 +65,4 @@ def _rotated_supported(query):
 # the rotated base: one pass of the HIP butterfly kernel around the plain launchers (reference
 # backends/triton/quant_rotated.py registers its fused and separate-pass pairs the same way)
 register_rotated_launchers("hip", *compose(fwd, dgrad, rotate_2d))
-registry.register("quant_linear_rotated", "hip", make_quant_linear_rotated("hip"), supports=requires(kinds=("hip",), archs=("gfx950",), extra=_rotated_supported))
+registry.register("quant_linear_rotated", "hip", make_quant_linear_rotated("hip"), supports=requires(kinds=("hip",), archs=("gfx950",), dtypes=HALF, extra=_rotated_supported))

@@ -1,108 +1,111 @@
-"""Regular-Hadamard rotation over groups of the last dim (ConvRot).
+"""Group Hadamard rotation (ConvRot): `x . blockdiag(H_g)` along the last axis, `g = 4^j`.
 
-H_g is the normalised Kronecker power of H4 = [[1,1,1,-1],[1,1,-1,1],[1,-1,1,1],[-1,1,1,1]] for
-g = 4^j: symmetric and involutory, entries +-2^-j (exact in fp16 / bf16). `group_hadamard(x, g)`
-is x times blockdiag(H_g) over the last dim, its own inverse and its own adjoint (so its
-backward is the rotation of the incoming gradient). On a GPU, bf16 / fp16 tensors go through the
-hand-written HIP butterfly kernel; everything else through torch ops. Interface follows
-reference `src/kohakumoss_kernels/hadamard.py:31-101` and the `group_hadamard` op of
-`backends/triton/hadamard.py:108-152`.
+`H_g` is the j-fold Kronecker power of the 4 x 4 matrix with ones everywhere but -1 on the
+anti-diagonal, scaled by `2^-j`: symmetric, its own inverse, every entry `+-2^-j` (exact in
+fp16 and bf16). So the rotation is its own backward: `d/dx (x R) = dy R`.
+
+On a gfx950 device 16-bit tensors go to the HIP butterfly kernel (`km_group_hadamard`);
+elsewhere 16-bit inputs multiply by `H_g` in their own dtype and other dtypes run the fp32
+butterflies (both as reference `src/kohakumoss_kernels/hadamard.py:31-101`).
 """
 
-from functools import cache
+from __future__ import annotations
+
+from functools import lru_cache
 
 import torch
 from torch import Tensor
 
-H4 = ((1, 1, 1, -1), (1, 1, -1, 1), (1, -1, 1, 1), (-1, 1, 1, 1))
 GROUPS = (4, 16, 64, 256, 1024)
 HALF = (torch.float16, torch.bfloat16)
+_SEED = ((1.0, 1.0, 1.0, -1.0), (1.0, 1.0, -1.0, 1.0), (1.0, -1.0, 1.0, 1.0), (-1.0, 1.0, 1.0, 1.0))
 
 
 def stages(group: int) -> int:
-    """j of g = 4^j; ValueError unless `group` is a power of 4 of at least 4."""
-    j, g = 0, int(group)
-    while g > 1 and g % 4 == 0:
-        g //= 4
-        j += 1
+    """`j` with `group == 4^j`, j >= 1; ValueError for anything else."""
+    g, j = int(group), 0
+    while g >= 4 and g % 4 == 0:
+        g, j = g // 4, j + 1
     if g != 1 or j == 0:
         raise ValueError(f"Hadamard group {group} is not a power of 4 >= 4")
     return j
 
 
 def check_group(x: Tensor, group: int) -> int:
-    """The stage count of `group`; ValueError when it does not divide x's last dim."""
     j = stages(group)
     if x.shape[-1] % group:
         raise ValueError(f"last dim {x.shape[-1]} is not a multiple of group {group}")
     return j
 
 
-@cache
-def _matrix(group: int, dtype: torch.dtype, device: torch.device) -> Tensor:
-    seed = torch.tensor(H4, dtype=torch.float32)
+@lru_cache(maxsize=None)
+def _matrix(group: int, dtype: torch.dtype, device: str) -> Tensor:
+    seed = torch.tensor(_SEED)
     h = seed
     for _ in range(stages(group) - 1):
         h = torch.kron(h, seed)
-    return (h / float(group) ** 0.5).to(device=device, dtype=dtype)
+    return (h / float(2 ** stages(group))).to(device=device, dtype=dtype)
 
 
 def hadamard_matrix(group: int, dtype: torch.dtype = torch.float32, device="cpu") -> Tensor:
-    """H_group [group, group] in `dtype` on `device` (cached; do not modify)."""
-    return _matrix(int(group), dtype, torch.device(device))
+    """`H_group` (a fresh copy the caller may modify)."""
+    return _matrix(int(group), dtype, str(torch.device(device))).clone()
 
 
-def _butterflies(x: Tensor, group: int, j: int) -> Tensor:
-    """j fp32 4-point stages, most significant base-4 digit first: y_k = sum(x) - 2 x_(3-k),
-    the sum taken in index order."""
-    v = x.float()
-    rows = v.numel() // group
-    for a in range(j):
-        x0, x1, x2, x3 = v.reshape(rows * 4**a, 4, group // 4 ** (a + 1)).unbind(1)
-        total = ((x0 + x1) + x2) + x3
-        v = torch.stack([total - 2.0 * x3, total - 2.0 * x2, total - 2.0 * x1, total - 2.0 * x0], 1)
-    return (v.reshape(x.shape) * 2.0**-j).to(x.dtype)
+def _butterflies(x: Tensor, group: int) -> Tensor:
+    """fp32 stages of 4-point butterflies, most significant base-4 digit of the index first:
+    with t = ((x0 + x1) + x2) + x3 the outputs are t - 2 x3, t - 2 x2, t - 2 x1, t - 2 x0."""
+    j = check_group(x, group)
+    v = x.to(torch.float32)
+    outer = v.numel() // group
+    for stage in range(j):
+        inner = group // 4 ** (stage + 1)
+        quad = v.reshape(outer * 4**stage, 4, inner)
+        total = ((quad[:, 0] + quad[:, 1]) + quad[:, 2]) + quad[:, 3]
+        v = torch.stack([total - 2.0 * quad[:, 3 - i] for i in range(4)], dim=1)
+    return (v.reshape(x.shape) * (0.5**j)).to(x.dtype)
 
 
 def group_hadamard_eager(x: Tensor, group: int) -> Tensor:
-    """x [..., K] -> x . blockdiag(H_group) in x's dtype with torch ops: a 16-bit matmul with H
-    (fp32 accumulation) for fp16 / bf16, fp32 butterflies for any other dtype."""
-    j = check_group(x, group)
+    check_group(x, group)
     if x.dtype in HALF:
-        return (x.reshape(-1, group) @ hadamard_matrix(group, x.dtype, x.device)).reshape(x.shape)
-    return _butterflies(x, group, j)
+        h = _matrix(int(group), x.dtype, str(x.device))
+        return (x.reshape(-1, group) @ h).reshape(x.shape)
+    return _butterflies(x, group)
 
 
 def rotate_2d(x: Tensor, group: int) -> Tensor:
-    """[R, K] -> [R, K] rotated, no autograd: the HIP kernel for 16-bit device tensors, torch ops
-    otherwise."""
+    """Rotation without autograd: the HIP kernel for 16-bit device tensors on gfx950, the eager
+    forms otherwise."""
     check_group(x, group)
-    if x.device.type == "cuda" and x.dtype in HALF:
-        from kohakumosstrainer_amd import native
+    if x.is_cuda and x.dtype in HALF:
+        from kohakumosstrainer_amd.kernels.arch import arch_of
 
-        return native.group_hadamard(x, group)
-    with torch.no_grad():
-        return group_hadamard_eager(x, group)
+        if arch_of(x.device).name == "gfx950":
+            from kohakumosstrainer_amd import native
 
-
-@torch.library.custom_op("kohakumoss_amd::group_hadamard", mutates_args=())
-def _op(x: Tensor, group: int) -> Tensor:
-    return rotate_2d(x, group)
+            return native.group_hadamard(x.reshape(-1, x.shape[-1]), group).reshape(x.shape)
+    return group_hadamard_eager(x, group)
 
 
-@_op.register_fake
-def _(x, group):
-    return torch.empty_like(x)
+_LIB = torch.library.Library("kohakumoss_amd", "FRAGMENT")
+_LIB.define("group_hadamard(Tensor x, int group) -> Tensor")
+torch.library.impl("kohakumoss_amd::group_hadamard", "CompositeExplicitAutograd", lib=_LIB)(lambda x, group: rotate_2d(x, group))
+torch.library.register_fake("kohakumoss_amd::group_hadamard", lib=_LIB)(lambda x, group: torch.empty_like(x))
 
 
 def _setup(ctx, inputs, output):
     ctx.group = inputs[1]
 
 
-_op.register_autograd(lambda ctx, g: (_op(g.contiguous(), ctx.group), None), setup_context=_setup)
+def _backward(ctx, grad):
+    return torch.ops.kohakumoss_amd.group_hadamard(grad.contiguous(), ctx.group), None
+
+
+torch.library.register_autograd("kohakumoss_amd::group_hadamard", _backward, setup_context=_setup, lib=_LIB)
 
 
 def group_hadamard(x: Tensor, group: int) -> Tensor:
-    """x [..., K] -> x . blockdiag(H_group), differentiable (the backward is the same rotation)."""
-    shape = x.shape
-    return _op(x.reshape(-1, shape[-1]).contiguous(), int(group)).view(shape)
+    """Differentiable `x . blockdiag(H_group)`; traces as one op under torch.compile."""
+    check_group(x, group)
+    return torch.ops.kohakumoss_amd.group_hadamard(x.contiguous(), int(group))

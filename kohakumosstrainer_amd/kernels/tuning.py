@@ -17,7 +17,10 @@ Mirrors the semantics of reference `src/kohakumoss_kernels/tuning/tuner.py` (`se
      calls), the winner is stored with every timing and failure, and settled.
 
 Table file: `<KOHAKUMOSS_KERNEL_CACHE or ~/.cache/kohakumoss_kernels>/tuning/<card key>/<tag>/<kernel>.json`,
-rows `{key: {"config", "timings_ms", "failures"}}`, merged on write and replaced atomically.
+rows `{key: {"config", "timings_ms", "failures"[, "working_mib"]}}`, merged on write and replaced
+atomically. `working_mib` is the peak device memory each timed candidate took beyond what was
+allocated before it ran; a candidate whose first run takes more than the caller's `working_bound`
+is dropped from the shortlist like one that fails to launch (reference `tuner.py:363-442`).
 """
 
 import hashlib
@@ -167,9 +170,12 @@ class TuneTable:
         row = self.rows.get(key)
         return None if row is None else row["config"]
 
-    def put(self, key: str, config: dict, timings: dict, failures: dict) -> None:
+    def put(self, key: str, config: dict, timings: dict, failures: dict, working_mib: dict | None = None) -> None:
+        row = {"config": config, "timings_ms": timings, "failures": failures}
+        if working_mib:
+            row["working_mib"] = working_mib
         with self.lock:
-            self.rows = {**(_read_json(self.path) or {}), **self.rows, key: {"config": config, "timings_ms": timings, "failures": failures}}
+            self.rows = {**(_read_json(self.path) or {}), **self.rows, key: row}
             _write_json_atomic(self.path, self.rows)
 
 
@@ -236,90 +242,149 @@ def _canon(config: dict) -> str:
     return json.dumps(config, sort_keys=True, default=str)
 
 
+class _Problem:
+    """One (device, kernel, key) and what `select` learns about it: shared bookkeeping of the
+    ways a configuration gets picked."""
+
+    def __init__(self, kernel: str, device: torch.device, key: str):
+        self.kernel, self.device, self.key = kernel, device, key
+        self.ident = (str(device), kernel, key)
+        self.errors: dict[str, str] = {}
+
+    def settle(self, config: dict) -> dict:
+        _chosen[self.ident] = config
+        DEFERRED.discard(self.ident)
+        return config
+
+    def give_up(self) -> ConfigsFailed:
+        err = ConfigsFailed(self.kernel, dict(self.errors), persist=all(_TOOLCHAIN_HINT(v) for v in self.errors.values()), problem=self.key)
+        _failed[self.ident] = err
+        return err
+
+    def try_once(self, config: dict, launch: Callable[[dict], Callable[[], object]]) -> Callable[[], object] | None:
+        """Build and run `config` once; None (and the reason noted) when it cannot."""
+        try:
+            run = launch(config)
+            run()
+            if self.device.type == "cuda":
+                torch.cuda.synchronize(self.device)
+            return run
+        except BUILD_ERRORS as err:
+            if isinstance(err, torch.OutOfMemoryError):
+                raise
+            self.errors[config_name(config)] = describe(err)
+            return None
+
+
+def _TOOLCHAIN_HINT(text: str) -> bool:
+    return is_toolchain_error(RuntimeError(text))
+
+
+def _peak_mib(device: torch.device) -> float:
+    return torch.cuda.max_memory_allocated(device) / 2**20 if device.type == "cuda" else 0.0
+
+
 def select(
     kernel: str,
     device: torch.device | str,
     key: str,
     candidates: Callable[[], Sequence[dict]],
-    launch: Callable[[dict], Callable[[], object]],
+    launch: Callable[[dict], Callable[[], object]] | None,
     shortlist: int = 4,
-    errors: tuple[type[BaseException], ...] = BUILD_ERRORS,
     in_backward: bool = False,
+    timing: Callable[[Callable[[], object], torch.device], float] | None = None,
+    working_bound: float | None = None,
 ) -> dict:
-    """The config for problem `key` of `kernel` on `device` (see the module docstring)."""
-    ident = (str(device), kernel, key)
-    chosen = _chosen.get(ident)
-    if chosen is not None:
-        return chosen
-    failed = _failed.get(ident)
-    if failed is not None:
-        raise ConfigsFailed(kernel, failed.errors, failed.persist, failed.problem)
+    """The configuration of `kernel` for problem `key` on `device`.
+
+    `candidates()` lists configurations, the planner's first pick first; `launch(config)` returns
+    a zero-argument callable that runs the kernel once on the caller's operands. `working_bound`
+    (MiB) drops candidates whose run allocates more than that. See the module docstring for the
+    order of the five cases."""
+    device = torch.device(device)
+    problem = _Problem(kernel, device, key)
+    if problem.ident in _chosen:
+        return _chosen[problem.ident]
+    if problem.ident in _failed:
+        raise _failed[problem.ident]
     ranked = list(candidates())
-    tab = table(kernel, device)
-    row = tab.get(key)
-    if row is not None:
-        match = [c for c in ranked if _canon(c) == _canon(row)]
-        if match:
-            _chosen[ident] = match[0]
-            return match[0]
-    if not timing_allowed(in_backward) or len(ranked) == 1:
-        if get_mode() == "off" or len(ranked) == 1:
-            _chosen[ident] = ranked[0]
-        return ranked[0]
+    if not ranked:
+        raise ConfigsFailed(kernel, {"candidates": "the planner offered none"}, persist=False, problem=key)
+
+    stored = table(kernel, device).get(key) if get_mode() == "table" else None
+    if stored is not None:
+        wanted = _canon(stored)
+        for config in ranked:
+            if _canon(config) == wanted:
+                return problem.settle(config)
+
+    if len(ranked) == 1:
+        return problem.settle(ranked[0])  # nothing to compare
+    if not timing_allowed(in_backward):
+        # nothing may be measured here: the planner's first pick serves, and only counts as the
+        # answer when no measurement will ever be made (mode off)
+        return problem.settle(ranked[0]) if get_mode() == "off" else ranked[0]
+
     if _state["frozen"] or _state["defer"]:
-        return _bind_untimed(ident, ranked, launch, errors)
+        DEFERRED.add(problem.ident)
+        for config in ranked:
+            if problem.try_once(config, launch) is not None:
+                return config  # provisional: timed once a tuning window opens
+        raise problem.give_up()
+
+    measure = timing or (lambda run, dev: best_ms(run, dev))
+    timings: dict[str, float] = {}
+    working: dict[str, float] = {}
+    by_name = {}
+    for config in ranked[: max(1, shortlist)]:
+        name = config_name(config)
+        if device.type == "cuda":
+            torch.cuda.synchronize(device)
+            torch.cuda.reset_peak_memory_stats(device)
+        before = torch.cuda.memory_allocated(device) / 2**20 if device.type == "cuda" else 0.0
+        run = problem.try_once(config, launch)
+        if run is None:
+            continue
+        took = max(0.0, _peak_mib(device) - before)
+        if device.type == "cuda":
+            working[name] = round(took, 3)
+        if working_bound is not None and took > working_bound:
+            problem.errors[name] = f"working memory {took:.1f} MiB exceeds the bound of {working_bound:.1f} MiB"
+            continue
+        try:
+            timings[name] = measure(run, device)
+        except BUILD_ERRORS as err:
+            if isinstance(err, torch.OutOfMemoryError):
+                raise
+            problem.errors[name] = describe(err)
+            continue
+        by_name[name] = config
+    if not timings:
+        # the shortlist is exhausted: anything further down that runs at all still serves
+        for config in ranked[max(1, shortlist) :]:
+            if problem.try_once(config, launch) is not None:
+                table(kernel, device).put(key, config, {}, dict(problem.errors))
+                return problem.settle(config)
+        raise problem.give_up()
     TIMED[kernel] = TIMED.get(kernel, 0) + 1
-    timings, failures, toolchain, best = {}, {}, [], None
-    for config in ranked[:shortlist]:
-        try:
-            with torch.enable_grad():
-                ms = best_ms(launch(config), device)
-        except torch.OutOfMemoryError:
-            raise
-        except errors as err:
-            failures[config_name(config)] = describe(err)[:300]
-            toolchain.append(is_toolchain_error(err))
-            continue
-        timings[config_name(config)] = ms
-        if best is None or ms < timings[config_name(best)]:
-            best = config
-    if best is None:
-        err = ConfigsFailed(kernel, failures, all(toolchain), f"{kernel}:{key}")
-        _failed[ident] = err
-        raise err
-    tab.put(key, best, timings, failures)
-    _chosen[ident] = best
-    return best
-
-
-def _bind_untimed(ident, ranked, launch, errors) -> dict:
-    failures, toolchain = {}, []
-    for config in ranked:
-        try:
-            with torch.enable_grad():
-                launch(config)()
-        except errors as err:
-            failures[config_name(config)] = describe(err)[:300]
-            toolchain.append(is_toolchain_error(err))
-            continue
-        _chosen[ident] = config
-        DEFERRED.add(ident)
-        return config
-    err = ConfigsFailed(ident[1], failures, all(toolchain), f"{ident[1]}:{ident[2]}")
-    _failed[ident] = err
-    raise err
+    winner = by_name[min(timings, key=timings.get)]
+    table(kernel, device).put(key, winner, timings, dict(problem.errors), working)
+    return problem.settle(winner)
 
 
 def forget(kernel: str, device: torch.device | str, key: str) -> None:
-    """Drop this process's choice for the problem (its config turned out unable to run)."""
-    _chosen.pop((str(device), kernel, key), None)
+    """Drop what this process settled for one problem (a stored row stays on disk)."""
+    ident = (str(torch.device(device)), kernel, key)
+    _chosen.pop(ident, None)
+    _failed.pop(ident, None)
+    DEFERRED.discard(ident)
 
 
 def settled(kernel: str, device: torch.device | str, key: str) -> dict | None:
-    chosen = _chosen.get((str(device), kernel, key))
-    return chosen if chosen is not None else table(kernel, device).get(key)
+    return _chosen.get((str(torch.device(device)), kernel, key))
 
 
 def decided(kernel: str, device: torch.device | str, key: str) -> bool:
-    """Whether `select` has a settled choice for this problem (callers bind only then)."""
-    return (str(device), kernel, key) in _chosen
+    """True once the choice for `key` will not change in this process: callers cache a bound
+    runner only then."""
+    return (str(torch.device(device)), kernel, key) in _chosen

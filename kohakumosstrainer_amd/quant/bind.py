@@ -1,5 +1,7 @@
-"""Binding quantized linears to their compute device and dtype after a placement (reference
-`src/kohakumoss/quant/bind.py:14-40`; W4A8 and embedding bases are outside this path)."""
+"""Re-binding the quantized bases of a model after it moved or changed dtype, and switching int8
+bases to the int8 compute linear. Replaces reference `src/kohakumoss/quant/bind.py`."""
+
+from __future__ import annotations
 
 import torch
 from torch import nn
@@ -8,26 +10,29 @@ from kohakumosstrainer_amd.quant.compute import ComputeWeight
 from kohakumosstrainer_amd.quant.weights import QuantWeight
 
 
+def work_device(device) -> torch.device:
+    """Where quantization work runs for a model headed to `device`: that device when it is a GPU
+    that is there, else the host."""
+    device = torch.device(device)
+    return device if device.type == "cuda" and torch.cuda.is_available() else torch.device("cpu")
+
+
 def rebind_quant(module: nn.Module, device, dtype, autograd: bool = True) -> None:
-    """Bind every quantized base to (device, dtype); `autograd=False` binds fp8-compute bases
-    of a model that never runs backward to the gradient-free op."""
-    for m in module.modules():
-        if isinstance(m, ComputeWeight):
-            m.bind(dtype, device, autograd=autograd)
-        elif isinstance(m, QuantWeight):
-            m.bind(dtype, device)
+    """Bind every quantized base under `module` for `(device, dtype)`: each resolves its op once
+    here instead of on its first call."""
+    for child in module.modules():
+        if isinstance(child, ComputeWeight):
+            child.bind(dtype, device, autograd=autograd)
+        elif isinstance(child, QuantWeight):
+            child.bind(dtype, device)
 
 
 def set_int8_compute(module: nn.Module, dgrad: str) -> int:
-    """Select int8 compute (the `int8_linear` op with input-gradient mode `dgrad`) on every int8
-    base inside `module`; it takes effect at their next `bind`. Returns how many were switched."""
-    switched = [m for m in module.modules() if isinstance(m, QuantWeight) and m.fmt == "int8"]
-    for m in switched:
-        m.int8_dgrad = dgrad
-    return len(switched)
-
-
-def work_device(device) -> torch.device:
-    """Where weights are quantized: the compute device when it is a GPU."""
-    device = torch.device(device)
-    return device if device.type == "cuda" else torch.device("cpu")
+    """Route every int8 weight-only base under `module` through the int8 compute linear with the
+    given input-gradient mode; returns how many were switched."""
+    switched = 0
+    for child in module.modules():
+        if isinstance(child, QuantWeight) and child.fmt == "int8":
+            child.int8_dgrad, child._call = dgrad, None
+            switched += 1
+    return switched

@@ -1,8 +1,16 @@
-"""Quantize the frozen linears of a model in place: weight-only (int8 / fp8, `QuantWeight`) or
-fp8 compute (fp8_compute / mxfp8, `ComputeWeight`); attach trainable fp8 compute caches.
-Mirrors reference `src/kohakumoss/quant/convert.py:29-244` without the checkpoint-source
-plumbing (weights are always quantized from the module's own parameter).
+"""Turning a model's linears into quantized ones.
+
+    make_base(w, fmt, ...)           a QuantWeight (int8 / fp8) or ComputeWeight (fp8_compute / mxfp8)
+    quantize_model(model, fmt, ...)  every accepted MossLinear gets a frozen base; returns a report
+    attach_compute(model, fmt, ...)  every accepted MossLinear keeps its weight and gets an fp8 cache
+    QuantLinear / quantize_torch_linears   the same for plain nn.Linear modules (text encoder)
+
+A layer is accepted when the filter says so (`default_filter`: not a kept-fp32 name, both sides at
+least `min_features`) and, for compute precisions, when its shape tiles by 128.
+Replaces reference `src/kohakumoss/quant/convert.py:29-244`.
 """
+
+from __future__ import annotations
 
 from collections.abc import Callable
 
@@ -10,28 +18,32 @@ import torch
 from torch import nn
 
 from kohakumosstrainer_amd.model.linear import MossLinear
+from kohakumosstrainer_amd.quant.bind import work_device as default_work_device
 from kohakumosstrainer_amd.quant.compute import COMPUTE, ComputeCache, ComputeWeight, eligible, recipe_of
-from kohakumosstrainer_amd.quant.weights import QuantWeight
+from kohakumosstrainer_amd.quant.weights import FORMATS, QuantWeight
+
+PRECISIONS = (*FORMATS, *COMPUTE)
 
 
 def make_base(w: torch.Tensor, fmt: str, recipe: str = "row", dgrad: bool = False):
-    """The quantized base of weight `w` under precision `fmt` (`recipe` and `dgrad` apply to
-    fp8_compute / mxfp8)."""
     if fmt in COMPUTE:
         return ComputeWeight.from_weight(w, recipe_of(fmt, recipe), dgrad)
-    return QuantWeight.from_weight(w, fmt)
+    if fmt in FORMATS:
+        return QuantWeight.from_weight(w, fmt)
+    raise ValueError(f"base precision {fmt!r} not in {PRECISIONS}")
 
 
 def accepts(fmt: str, out_features: int, in_features: int) -> bool:
-    """Whether a [N, K] weight can take `fmt` (fp8 compute needs aligned shapes)."""
+    """Shape rule of a precision: compute bases need both sides to tile by 128."""
     return fmt not in COMPUTE or eligible(out_features, in_features) is None
 
 
 def default_filter(keep_fp32: tuple[str, ...], min_features: int = 256) -> Callable[[str, nn.Linear], bool]:
-    """Quantize every linear except those under a kept name and small ones."""
+    """Accept a linear unless its name contains one of `keep_fp32` or it is narrower than
+    `min_features` on either side."""
 
     def accept(name: str, lin: nn.Linear) -> bool:
-        if any(name == k or name.startswith(k + ".") for k in keep_fp32):
+        if any(part in name for part in keep_fp32):
             return False
         return min(lin.in_features, lin.out_features) >= min_features
 
@@ -39,86 +51,95 @@ def default_filter(keep_fp32: tuple[str, ...], min_features: int = 256) -> Calla
 
 
 class QuantLinear(nn.Module):
-    """Inference replacement of a plain nn.Linear by a quantized weight (+ bias)."""
+    """A plain `nn.Linear` replaced by a quantized base and its (dense) bias."""
 
     def __init__(self, linear: nn.Linear, fmt: str, compute_dtype: torch.dtype, recipe: str = "row", work_device=None):
         super().__init__()
-        self.in_features, self.out_features = linear.in_features, linear.out_features
-        home = linear.weight.device
-        self.qweight = make_base(linear.weight.detach().to(work_device or home), fmt, recipe).to(home)
-        self.qweight.bind(compute_dtype)
-        self.bias = None if linear.bias is None else nn.Parameter(linear.bias.detach(), requires_grad=False)
+        where = linear.weight.device if work_device is None else torch.device(work_device)
+        base = make_base(linear.weight.detach().to(where), fmt, recipe).to(linear.weight.device)
+        self._adopt(linear.in_features, linear.out_features, base, linear.bias, compute_dtype)
+
+    def _adopt(self, in_features, out_features, base, bias, compute_dtype) -> None:
+        self.in_features, self.out_features, self.compute_dtype = in_features, out_features, compute_dtype
+        self.base = base
+        self.bias = None if bias is None else nn.Parameter(bias.detach().clone(), requires_grad=False)
 
     @classmethod
     def from_base(cls, in_features: int, out_features: int, base, bias, compute_dtype: torch.dtype) -> "QuantLinear":
-        """A QuantLinear over an already-quantized base."""
         self = cls.__new__(cls)
         nn.Module.__init__(self)
-        self.in_features, self.out_features = in_features, out_features
-        self.qweight = base
-        self.qweight.bind(compute_dtype)
-        self.bias = None if bias is None else nn.Parameter(bias, requires_grad=False)
+        self._adopt(in_features, out_features, base, bias, compute_dtype)
         return self
 
     def forward(self, x):
-        return self.qweight.linear(x, None if self.bias is None else self.bias.to(x.dtype))
+        bias = None if self.bias is None else self.bias.to(x.dtype)
+        return self.base.linear(x, bias)
+
+
+def _walk_children(module: nn.Module, prefix: str = ""):
+    for name, child in module.named_children():
+        path = f"{prefix}.{name}" if prefix else name
+        yield module, name, path, child
+        yield from _walk_children(child, path)
 
 
 @torch.no_grad()
 def quantize_torch_linears(module: nn.Module, fmt: str, compute_dtype: torch.dtype, min_features: int = 256) -> int:
-    """Replace every large plain nn.Linear inside `module` (e.g. a frozen text encoder);
-    returns how many."""
-    count = 0
-    for name, child in list(module.named_children()):
-        big = type(child) is nn.Linear and min(child.in_features, child.out_features) >= min_features
-        if big and accepts(fmt, child.out_features, child.in_features):
-            setattr(module, name, QuantLinear(child, fmt, compute_dtype))
-            count += 1
-        elif not big:
-            count += quantize_torch_linears(child, fmt, compute_dtype, min_features)
-    return count
+    """Replace every plain `nn.Linear` under `module` that passes the size and shape rules by a
+    `QuantLinear`; returns how many were replaced."""
+    accept = default_filter((), min_features)
+    swaps = [(parent, name, child) for parent, name, path, child in _walk_children(module)
+             if type(child) is nn.Linear and accept(path, child) and accepts(fmt, child.out_features, child.in_features)]
+    for parent, name, child in swaps:
+        setattr(parent, name, QuantLinear(child, fmt, compute_dtype))
+    return len(swaps)
+
+
+def _accepted(model: nn.Module, fmt: str, accept) -> tuple[list[tuple[str, MossLinear]], int]:
+    taken, skipped = [], 0
+    for path, layer in model.named_modules():
+        if not isinstance(layer, MossLinear) or not layer.is_plain:
+            continue
+        if accept is not None and not accept(path, layer):
+            continue
+        if accepts(fmt, layer.out_features, layer.in_features):
+            taken.append((path, layer))
+        else:
+            skipped += 1
+    return taken, skipped
 
 
 @torch.no_grad()
 def attach_compute(model: nn.Module, fmt: str, accept, compute_dtype: torch.dtype, recipe: str = "row", dgrad: bool = True) -> list[MossLinear]:
-    """Trainable fp8 compute: a ComputeCache, quantized from the current weight, on every
-    accepted dense MossLinear of an fp8-compute shape; returns those linears (their caches
-    need `refresh` after every optimizer step)."""
-    out = []
-    for name, lin in list(model.named_modules()):
-        if not isinstance(lin, MossLinear) or lin.base is not None:
-            continue
-        if not accept(name, lin) or not accepts(fmt, lin.out_features, lin.in_features):
-            continue
+    """Give every accepted trainable MossLinear an fp8 cache of its weight (quantized now; the
+    trainer refreshes it after each optimizer step). Returns the layers that got one."""
+    if fmt not in COMPUTE:
+        raise ValueError(f"compute precision {fmt!r} not in {COMPUTE}")
+    taken, _ = _accepted(model, fmt, accept)
+    for _, layer in taken:
         cache = ComputeCache(recipe_of(fmt, recipe), dgrad)
-        cache.refresh(lin.weight)
-        cache.bind(compute_dtype, lin.weight.device)
-        lin.set_compute(cache)
-        out.append(lin)
-    return out
+        cache.refresh(layer.weight)
+        cache.bind(compute_dtype, layer.weight.device)
+        layer.set_compute(cache)
+    return [layer for _, layer in taken]
 
 
 @torch.no_grad()
-def quantize_model(model: nn.Module, fmt: str, accept=None, compute_dtype: torch.dtype | None = None, recipe: str = "row", dgrad: bool = False, work_device=None) -> dict[str, int]:
-    """Replace accepted dense MossLinear bases with QuantWeight (int8 / fp8) or ComputeWeight
-    (fp8_compute / mxfp8), quantizing on `work_device` (default: where the weight is); the dense
-    parameter becomes an empty placeholder. Returns counts and bytes (`skipped`: accepted
-    layers whose shape fp8 compute cannot take)."""
-    accept = accept or default_filter(())
-    report = {"layers": 0, "dense_bytes": 0, "quant_bytes": 0, "skipped": 0}
-    for name, lin in list(model.named_modules()):
-        if not isinstance(lin, MossLinear) or lin.base is not None or not accept(name, lin):
-            continue
-        if not accepts(fmt, lin.out_features, lin.in_features):
-            report["skipped"] += 1
-            continue
-        w = lin.weight.detach()
-        home = w.device
-        base = make_base(w.to(work_device or home), fmt, recipe, dgrad).to(home)
-        report["layers"] += 1
-        report["dense_bytes"] += w.nbytes
-        report["quant_bytes"] += base.nbytes()
-        lin.weight = nn.Parameter(torch.empty(0, dtype=w.dtype, device=home), requires_grad=False)
-        lin.set_base(base)
-        base.bind(compute_dtype or w.dtype)
-    return report
+def quantize_model(model: nn.Module, fmt: str, accept=None, compute_dtype: torch.dtype | None = None, recipe: str = "row", dgrad: bool = False, work_device=None) -> dict:
+    """Swap the weight of every accepted MossLinear for a frozen base. Quantization runs on
+    `work_device` (default: the layer's own device if it is a GPU); the base ends up where the
+    layer was. Report: layers converted, layers skipped for their shape, bytes before / after."""
+    if fmt not in PRECISIONS:
+        raise ValueError(f"base precision {fmt!r} not in {PRECISIONS}")
+    taken, skipped = _accepted(model, fmt, accept if accept is not None else default_filter(()))
+    dense_bytes = quant_bytes = 0
+    for _, layer in taken:
+        home = layer.weight.device
+        where = default_work_device(home) if work_device is None else torch.device(work_device)
+        dense_bytes += layer.weight.numel() * layer.weight.element_size()
+        base = make_base(layer.weight.detach().to(where), fmt, recipe, dgrad).to(home)
+        quant_bytes += base.nbytes()
+        layer.set_base(base)
+        if compute_dtype is not None:
+            base.bind(compute_dtype, home)
+    return {"layers": len(taken), "skipped": skipped, "dense_bytes": dense_bytes, "quant_bytes": quant_bytes, "format": fmt}

@@ -160,7 +160,9 @@ def save_quantized(model: nn.Module, path: str | Path, dtype: torch.dtype = torc
         if f"{p}.weight" not in keys:
             keys.append(f"{p}.weight")
     state, meta = quantized_state(model, keys, dtype)
-    save_file({k: (v.view(torch.uint8) if v.dtype == torch.float8_e4m3fn else v) for k, v in state.items()}, str(path), metadata=meta)
+    # the codes keep their float8_e4m3fn dtype in the file: a reader that hands `<path>.weight`
+    # straight to its fp8 GEMM (the reference's `attach_stored`) must not see bytes
+    save_file(state, str(path), metadata=meta)
     return json.loads(meta[FP8_KEY])
 
 
@@ -168,18 +170,35 @@ def save_quantized(model: nn.Module, path: str | Path, dtype: torch.dtype = torc
 def load_quantized(model: nn.Module, path: str | Path, device, dtype: torch.dtype) -> int:
     """Load a file written by `save_quantized` (or by the reference's exporter) into `model`:
     recorded layers get their fp8 bases from the file, every other tensor is loaded as usual.
-    Returns the number of attached layers (0 for a file without a record: plain load)."""
+    Returns the number of attached layers (0 for a file without a record: plain load).
+
+    The dense parameter of a recorded layer is replaced by an empty placeholder before anything
+    moves to `device`, so its 16-bit weight is never materialised there (and a model built on the
+    meta device loads). Every other parameter and persistent buffer of the model must be in the
+    file and the file must hold nothing else: a missing or misspelt tensor raises KeyError instead
+    of leaving an initial value in place. Codes stored as bytes by an earlier version of this
+    package are reinterpreted as e4m3."""
     from safetensors import safe_open
 
     record = read_record(path)
+    device = torch.device(device)
     with safe_open(str(path), framework="pt", device="cpu") as f:
         names = set(f.keys())
         weights, scales = stored_keys(record) if record else (set(), set())
-        missing = (weights | scales) - names
-        if missing:
-            raise KeyError(f"{path}: the record names tensors the file lacks: {sorted(missing)[:4]}")
+        absent = (weights | scales) - names
+        if absent:
+            raise KeyError(f"{path}: the record names tensors the file lacks: {sorted(absent)[:4]}")
+        for key in sorted(weights):
+            layer = model.get_submodule(key.removesuffix(".weight"))
+            if not isinstance(layer, MossLinear):
+                raise TypeError(f"{key}: {type(layer).__name__} is not a MossLinear")
+            layer.weight = nn.Parameter(torch.empty(0, dtype=dtype, device=device), requires_grad=False)
         plain = {k: f.get_tensor(k) for k in names - weights - scales}
-        model.load_state_dict(plain, strict=False)
+        on_meta = any(t.is_meta for t in list(model.parameters()) + list(model.buffers()))
+        result = model.load_state_dict(plain, strict=False, assign=on_meta)
+        missing = sorted(set(result.missing_keys) - weights)
+        if missing or result.unexpected_keys:
+            raise KeyError(f"{path} does not match the model: missing {missing[:4]}, unexpected {sorted(result.unexpected_keys)[:4]}")
         model.to(device)
         if not record:
             return 0

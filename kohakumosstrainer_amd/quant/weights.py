@@ -1,138 +1,120 @@
-"""Quantized frozen base weights (per-output-row scales) as MossLinear base storage.
+"""Weight-only quantized frozen bases: int8 or e4m3 codes with one fp32 scale per output row.
 
-int8: q = round(w / s) clamped to [-127, 127], s = max|w_row| / 127.
-fp8 (e4m3fn): q = fp8(w / s), s = max|w_row| / 448.
-`linear` is bound once per (device, dtype): on the host the plain-op composition (dequantize,
-then a dense linear, saving only `q` / `scale` for the input gradient); on a GPU the
-`quant_linear` op the registry resolves (the HIP dequant-GEMM on gfx950) or, for an int8 base
-with `int8_dgrad` set (int8 compute), the `int8_linear` op (activations quantized per row, int8
-MFMA GEMM). `rotation` > 0 marks a ConvRot base: the stored codes are those of W R with
-R = blockdiag(H_rotation) over K, and the linear rotates x first (`quant_linear_rotated`, or the
-`group` of `int8_linear`). Mirrors reference `src/kohakumoss/quant/weights.py:31-140,159-202`.
+    quantize(w, fmt)          -> (q [N, K], scale [N])
+    QuantWeight               a module holding them; `linear(x, bias)` = x @ (q * scale)^T + bias
+
+`rotation` > 0 marks codes of `W R` (R the group Hadamard of that size: ConvRot files); the
+linear then rotates x. `int8_dgrad` set ("int8" or "16bit") routes an int8 base through the int8
+*compute* linear instead (activations quantized per row, integer GEMM). On the host the linear is
+plain torch with a custom backward that keeps only `(q, scale)` alive; on a GPU it is the
+registry's op. Replaces reference `src/kohakumoss/quant/weights.py:31-190`.
 """
 
-from functools import partial
+from __future__ import annotations
 
 import torch
-import torch.nn.functional as F
 from torch import Tensor, nn
 
-from kohakumosstrainer_amd.kernels import registry
+from kohakumosstrainer_amd.kernels import hadamard, registry
 
-FP8_MAX = 448.0
-INT8_MAX = 127.0
 FORMATS = ("int8", "fp8")
+_LIMIT = {"int8": 127.0, "fp8": 448.0}
+_FLOOR = 1e-12
 
 
 def quantize(w: Tensor, fmt: str) -> tuple[Tensor, Tensor]:
-    """`(q, scale[out])` of a 2-D weight; scale is fp32."""
-    v = w.detach().float()
-    amax = v.abs().amax(dim=1).clamp_min(1e-12)
+    """Per-output-row symmetric quantizer. The scale is `max(amax, 1e-12) / limit` with the limit
+    a Python number (127 for int8: codes round half to even; 448 for e4m3: one rounding of w / s)."""
+    if fmt not in FORMATS:
+        raise ValueError(f"quant format {fmt!r} not in {FORMATS}")
+    v = w.detach().to(torch.float32)
+    scale = v.abs().amax(dim=1).clamp_min(_FLOOR) / _LIMIT[fmt]
+    ratio = v / scale.unsqueeze(1)
     if fmt == "int8":
-        scale = amax / INT8_MAX
-        return torch.round(v / scale[:, None]).clamp_(-INT8_MAX, INT8_MAX).to(torch.int8), scale
-    if fmt == "fp8":
-        scale = amax / FP8_MAX
-        return (v / scale[:, None]).clamp_(-FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn), scale
-    raise ValueError(f"quant format {fmt!r} not in {FORMATS}")
+        return torch.round(ratio).clamp_(-127.0, 127.0).to(torch.int8), scale
+    return ratio.clamp_(-448.0, 448.0).to(torch.float8_e4m3fn), scale
 
 
 def dequantize(q: Tensor, scale: Tensor, dtype: torch.dtype) -> Tensor:
-    return (q.to(torch.float32) * scale.float()[:, None]).to(dtype)
+    return (q.to(torch.float32) * scale.to(torch.float32).unsqueeze(1)).to(dtype)
+
+
+class _HostLinear(torch.autograd.Function):
+    """x @ dequant(q, scale)^T on the host. The dequantized weight is rebuilt in backward: the
+    graph holds the codes and the scale, never a 16-bit matrix."""
+
+    @staticmethod
+    def forward(ctx, x, q, scale, bias):
+        ctx.save_for_backward(q, scale)
+        ctx.bias_dtype = None if bias is None else bias.dtype
+        return torch.nn.functional.linear(x, dequantize(q, scale, x.dtype), None if bias is None else bias.to(x.dtype))
+
+    @staticmethod
+    def backward(ctx, grad):
+        q, scale = ctx.saved_tensors
+        dx = grad @ dequantize(q, scale, grad.dtype) if ctx.needs_input_grad[0] else None
+        db = None
+        if ctx.bias_dtype is not None and ctx.needs_input_grad[3]:
+            db = grad.reshape(-1, grad.shape[-1]).to(torch.float32).sum(0).to(ctx.bias_dtype)
+        return dx, None, None, db
 
 
 class QuantWeight(nn.Module):
-    """BaseWeight holding `q` and `scale` as buffers (they follow `.to(device)`); `int8_dgrad`
-    is None (weight-only) or the input-gradient mode of int8 compute ("int8" | "16bit")."""
+    """Codes and scales of a frozen weight as buffers, and the way to multiply by them."""
 
     def __init__(self, q: Tensor, scale: Tensor, fmt: str, rotation: int = 0, int8_dgrad: str | None = None):
         super().__init__()
         if fmt not in FORMATS:
             raise ValueError(f"quant format {fmt!r} not in {FORMATS}")
+        if rotation:
+            hadamard.stages(rotation)
         if int8_dgrad is not None and fmt != "int8":
-            raise ValueError("int8 compute needs an int8 base")
-        self.fmt = fmt
-        self.rotation = int(rotation)
-        self.int8_dgrad = int8_dgrad
+            raise ValueError("the int8 compute linear needs an int8 base")
+        self.fmt, self.rotation, self.int8_dgrad = fmt, int(rotation), int8_dgrad
         self.register_buffer("q", q)
-        self.register_buffer("scale", scale.float())
-        self.shape = q.shape
-        self._linear = _host_linear
+        self.register_buffer("scale", scale.to(torch.float32))
+        self._call = None
+        self._bound_for = None
 
     @classmethod
     def from_weight(cls, w: Tensor, fmt: str) -> "QuantWeight":
         return cls(*quantize(w, fmt), fmt)
 
     def weight(self, dtype: torch.dtype) -> Tensor:
-        """W in `dtype` (the rotation undone: W = (q * s) R, R its own inverse)."""
-        if not self.rotation:
-            return dequantize(self.q, self.scale, dtype)
-        from kohakumosstrainer_amd.kernels.hadamard import group_hadamard_eager
-
-        return group_hadamard_eager(dequantize(self.q, self.scale, torch.float32), self.rotation).to(dtype)
+        """The dense weight this base stands for (rotated back when the codes are of W R)."""
+        dense = dequantize(self.q, self.scale, torch.float32)
+        if self.rotation:
+            dense = hadamard.group_hadamard_eager(dense, self.rotation)  # R is its own inverse
+        return dense.to(dtype)
 
     def materialize(self) -> Tensor:
         return self.weight(torch.float32)
 
     def bind(self, dtype: torch.dtype, device=None) -> None:
-        """Bind `linear` for (device, dtype) once."""
-        device = self.q.device if device is None else torch.device(device)
-        if device.type == "cpu":
-            self._linear = _host_linear
-            return
+        """Pick how `linear` runs for `(device, dtype)`, once."""
+        device = torch.device(device) if device is not None else self.q.device
+        self._bound_for = (device, dtype)
         if self.int8_dgrad is not None:
-            kernel = registry.resolve("int8_linear", device, dtype, group=self.rotation, dgrad=self.int8_dgrad)
-            self._linear = partial(_int8_linear, kernel)
-            return
+            op = registry.resolve("int8_linear", device, dtype, group=self.rotation, dgrad=self.int8_dgrad)
+            self._call = lambda x, bias: op(x, self.q, self.scale, bias, self.rotation, self.int8_dgrad)
+        elif device.type == "cpu":
+            self._call = self._on_host
+        elif self.rotation:
+            op = registry.resolve("quant_linear_rotated", device, dtype, fmt=self.fmt, group=self.rotation)
+            self._call = lambda x, bias: op(x, self.q, self.scale, bias, self.fmt, self.rotation)
+        else:
+            op = registry.resolve("quant_linear", device, dtype, fmt=self.fmt)
+            self._call = lambda x, bias: op(x, self.q, self.scale, bias, self.fmt)
+
+    def _on_host(self, x: Tensor, bias: Tensor | None) -> Tensor:
         if self.rotation:
-            kernel = registry.resolve("quant_linear_rotated", device, dtype, fmt=self.fmt, group=self.rotation)
-            self._linear = partial(_rotated_linear, kernel)
-            return
-        kernel = registry.resolve("quant_linear", device, dtype, fmt=self.fmt)
-        self._linear = partial(_kernel_linear, kernel)
+            x = hadamard.group_hadamard(x, self.rotation)
+        return _HostLinear.apply(x, self.q, self.scale, bias)
 
     def linear(self, x: Tensor, bias: Tensor | None) -> Tensor:
-        """x W^T (+ bias) through the bound implementation."""
-        return self._linear(self, x, bias)
+        if self._call is None or self._bound_for != (x.device, x.dtype):
+            self.bind(x.dtype, x.device)
+        return self._call(x, bias)
 
     def nbytes(self) -> int:
-        return self.q.nbytes + self.scale.numel() * 4
-
-
-class _HostLinear(torch.autograd.Function):
-    """Dequantize for this call, dense linear; only `q` / `scale` are saved."""
-
-    @staticmethod
-    def forward(ctx, x, q, scale, bias):
-        ctx.save_for_backward(q, scale)
-        ctx.bias_dtype = None if bias is None else bias.dtype
-        return F.linear(x, dequantize(q, scale, x.dtype), None if bias is None else bias.to(x.dtype))
-
-    @staticmethod
-    def backward(ctx, grad):
-        q, scale = ctx.saved_tensors
-        gx = grad @ dequantize(q, scale, grad.dtype) if ctx.needs_input_grad[0] else None
-        gb = grad.float().sum(0).to(ctx.bias_dtype) if ctx.bias_dtype is not None and ctx.needs_input_grad[3] else None
-        return gx, None, None, gb
-
-
-def _host_linear(qw: QuantWeight, x: Tensor, bias: Tensor | None) -> Tensor:
-    if qw.rotation:
-        from kohakumosstrainer_amd.kernels.rotated import quant_linear_rotated_eager
-
-        return quant_linear_rotated_eager(x, qw.q, qw.scale, bias, qw.fmt, qw.rotation)
-    lead = x.shape[:-1]
-    y = _HostLinear.apply(x.reshape(-1, x.shape[-1]), qw.q, qw.scale, bias)
-    return y.reshape(*lead, qw.q.shape[0])
-
-
-def _kernel_linear(kernel, qw: QuantWeight, x: Tensor, bias: Tensor | None) -> Tensor:
-    return kernel(x, qw.q, qw.scale, bias, qw.fmt)
-
-
-def _rotated_linear(kernel, qw: QuantWeight, x: Tensor, bias: Tensor | None) -> Tensor:
-    return kernel(x, qw.q, qw.scale, bias, qw.fmt, qw.rotation)
-
-
-def _int8_linear(kernel, qw: QuantWeight, x: Tensor, bias: Tensor | None) -> Tensor:
-    return kernel(x, qw.q, qw.scale, bias, qw.rotation, qw.int8_dgrad)
+        return sum(t.numel() * t.element_size() for t in (self.q, self.scale))

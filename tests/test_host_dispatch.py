@@ -37,7 +37,7 @@ def fake_ops():
     yield calls
     registry.reset_priority()
     registry.clear_failures()
-    registry._T.impls.pop("fake_op", None)
+    registry.unregister("fake_op")
 
 
 def test_arch_table():

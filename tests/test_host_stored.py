@@ -98,19 +98,77 @@ def test_plain_file_loads_without_a_record(tmp_path):
     assert torch.equal(fresh.a.weight, m.a.weight)
 
 
+ALL_KEYS = ["a.weight", "a.bias", "b.weight", "small.weight", "small.bias", "norm.weight", "norm.bias"]
+
+
 def test_record_naming_absent_tensors_or_wrong_shapes_fails(tmp_path):
     from safetensors.torch import save_file
 
     m = quantized_model("row")
-    state, meta = stored.quantized_state(m, ["a.weight", "a.bias", "b.weight"], torch.float32)
-    as_bytes = {k: (v.view(torch.uint8) if v.dtype == torch.float8_e4m3fn else v) for k, v in state.items()}
-    broken = dict(as_bytes)
+    state, meta = stored.quantized_state(m, ALL_KEYS, torch.float32)
+    broken = dict(state)
     del broken["b.weight_scale"]
     save_file(broken, str(tmp_path / "lacks.safetensors"), metadata=meta)
-    with pytest.raises(KeyError):
+    with pytest.raises(KeyError, match="record names"):
         stored.load_quantized(Tiny(), tmp_path / "lacks.safetensors", "cpu", torch.float32)
-    wrong = dict(as_bytes)
+    wrong = dict(state)
     wrong["a.weight"] = wrong["a.weight"][:64].contiguous()
     save_file(wrong, str(tmp_path / "shape.safetensors"), metadata=meta)
     with pytest.raises(ValueError, match="stored codes"):
         stored.load_quantized(Tiny(), tmp_path / "shape.safetensors", "cpu", torch.float32)
+
+
+def test_a_missing_or_misspelt_plain_tensor_is_an_error(tmp_path):
+    """Nothing of the model may silently keep its initial value, and the file may hold nothing the
+    model does not know."""
+    from safetensors.torch import save_file
+
+    m = quantized_model("mx")
+    state, meta = stored.quantized_state(m, ALL_KEYS, torch.float32)
+    short = {k: v for k, v in state.items() if k != "small.bias"}
+    save_file(short, str(tmp_path / "short.safetensors"), metadata=meta)
+    with pytest.raises(KeyError, match="small.bias"):
+        stored.load_quantized(Tiny(), tmp_path / "short.safetensors", "cpu", torch.float32)
+    extra = dict(state)
+    extra["smal.bias"] = state["small.bias"].clone()
+    save_file(extra, str(tmp_path / "extra.safetensors"), metadata=meta)
+    with pytest.raises(KeyError, match="smal.bias"):
+        stored.load_quantized(Tiny(), tmp_path / "extra.safetensors", "cpu", torch.float32)
+
+
+@pytest.mark.parametrize("codes_as", ("e4m3", "bytes"))
+def test_file_in_the_exporters_layout_loads(tmp_path, codes_as):
+    """A file laid out as the reference's exporter writes it (`quantized_state` ->
+    safetensors): codes under `<path>.weight` in float8_e4m3fn, scales under
+    `<path>.weight_scale`, the record in the metadata. Files of an earlier version of this package
+    (codes as bytes) load too. What `save_quantized` writes has the e4m3 dtype in the file."""
+    from safetensors import safe_open
+    from safetensors.torch import save_file
+
+    m = quantized_model("mx", seed=3)
+    state, meta = stored.quantized_state(m, ALL_KEYS, torch.bfloat16)
+    assert state["a.weight"].dtype == torch.float8_e4m3fn
+    if codes_as == "bytes":
+        state = {k: (v.view(torch.uint8) if v.dtype == torch.float8_e4m3fn else v) for k, v in state.items()}
+    save_file(state, str(tmp_path / "ref.safetensors"), metadata=meta)
+    fresh = Tiny()
+    assert stored.load_quantized(fresh, tmp_path / "ref.safetensors", "cpu", torch.bfloat16) == 2
+    assert torch.equal(fresh.a.base.q.view(torch.uint8), m.a.base.q.view(torch.uint8)) and fresh.a.base.q.dtype == torch.float8_e4m3fn
+    assert torch.equal(fresh.b.base.scale, m.b.base.scale)
+    stored.save_quantized(m, tmp_path / "ours.safetensors", torch.bfloat16)
+    with safe_open(str(tmp_path / "ours.safetensors"), framework="pt") as f:
+        assert f.get_tensor("a.weight").dtype == torch.float8_e4m3fn
+
+
+def test_meta_initialised_model_loads_without_dense_copies(tmp_path):
+    m = quantized_model("row", seed=4)
+    stored.save_quantized(m, tmp_path / "m.safetensors", torch.float32)
+    with torch.device("meta"):
+        empty = Tiny.__new__(Tiny)
+        nn.Module.__init__(empty)
+        empty.a, empty.b, empty.small, empty.norm = MossLinear(256, 128, bias=True), MossLinear(128, 256, bias=False), MossLinear(128, 8), nn.LayerNorm(8)
+    assert empty.a.weight.is_meta
+    assert stored.load_quantized(empty, tmp_path / "m.safetensors", "cpu", torch.float32) == 2
+    assert empty.a.weight.numel() == 0 and not any(p.is_meta for p in empty.parameters())
+    x = torch.randn(3, 256)
+    assert torch.equal(empty(x), m(x))
