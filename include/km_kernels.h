@@ -24,6 +24,7 @@ extern "C" {
 enum { KM_OK = 0, KM_ERR_ARG = -1, KM_ERR_LAUNCH = -2, KM_ERR_UNSUPPORTED = -3 };
 enum { KM_BF16 = 0, KM_F16 = 1, KM_F32 = 2 };          /* 16-bit activation / output dtypes */
 enum { KM_Q_INT8 = 0, KM_Q_E4M3 = 1 };                  /* weight-only code formats */
+enum { KM_WSCALE_ROWS = 0, KM_WSCALE_E8M0 = 1, KM_WSCALE_BLOCKS = 2 }; /* weight scale layouts of km_wo_gemm_dgrad_w16 */
 enum { KM_SCALES_ROWMAJOR = 0, KM_SCALES_PACKED = 1, KM_SCALES_KMAJOR = 2 };  /* scale layouts the GEMMs read */
 enum { KM_KERNEL_GEMM_MX = 0, KM_KERNEL_GEMM_FP8 = 1, KM_KERNEL_WO_FWD = 2, KM_KERNEL_WO_DGRAD = 3, KM_KERNEL_GEMM_BLOCKS = 4 };
 enum { KM_ROLE_ACT = 0, KM_ROLE_WEIGHT = 1 };                     /* operand roles of the block recipe */
@@ -183,6 +184,21 @@ int km_wo_gemm_fwd(const void *x, const void *q, const float *scale, const void 
 int km_wo_gemm_dgrad(const void *dy, const void *q, const float *scale, void *dx,
                      void *q_t_workspace, int64_t M, int64_t N, int64_t K, int q_format, int dtype,
                      int config, void *stream);
+
+/* Input gradient over the codes as they are stored, for int8 / e4m3 weight-only bases and for
+ * fp8 compute bases that keep no transposed copy: dx[M,K] = dy[M,N] @ round_dtype(q[N,K] * s(n,k)),
+ * the scaled weight rounded once to the activation dtype. The kernel transposes 8 x 4 bytes of
+ * codes in registers on their way to LDS: no workspace, no transposed copy, nothing allocated.
+ *   KM_WSCALE_ROWS    scale fp32 [N] (scale_ld 1) or one fp32 for the whole tensor (scale_ld 0)
+ *   KM_WSCALE_E8M0    scale uint8 [N, scale_ld] biased exponents, one per 32 codes of a row (MX);
+ *                     e4m3 codes only
+ *   KM_WSCALE_BLOCKS  scale fp32 [ceil(N/128), scale_ld], one per 128 x 128 block; e4m3 codes only
+ * Replaces Triton _dgrad_kernel (backends/triton/quant.py:80-129) and the 16-bit input gradient
+ * `dy @ dequantize(q, scale)` of an fp8 base (backends/triton/fp8/linear.py:152-153 over
+ * fp8/formats.py:103-126). */
+int km_wo_gemm_dgrad_w16(const void *dy, const void *q, const void *scale, int scale_kind,
+                         int64_t scale_ld, void *dx, int64_t M, int64_t N, int64_t K, int q_format,
+                         int dtype, int config, void *stream);
 
 /* km_wo_gemm_dgrad without a workspace argument and without any allocation: the transposed codes
  * go to a static device array of KM_WO_DGRAD_STATIC_MAX_CODES bytes that the library holds on every

@@ -18,7 +18,7 @@ CSRC = PKG / "csrc"
 OUT_DIR = PKG / "_lib"
 LIB = OUT_DIR / "libkm_kernels.so"
 HOST_LIB = OUT_DIR / "libkm_hostcheck.so"
-SOURCES = ("km_api.hip", "km_quant.hip", "km_gemm_fp8.hip", "km_gemm_fp8_w32.hip", "km_gemm_blocks.hip", "km_gemm_fused.hip", "km_wo_gemm.hip", "km_hadamard.hip")
+SOURCES = ("km_api.hip", "km_quant.hip", "km_gemm_fp8.hip", "km_gemm_fp8_w32.hip", "km_gemm_blocks.hip", "km_gemm_fused.hip", "km_wo_gemm.hip", "km_wo_dgrad.hip", "km_wo_fwd_bf16.hip", "km_wo_fwd_f16.hip", "km_wo_dgrad_bf16.hip", "km_wo_dgrad_f16.hip", "km_hadamard.hip")
 ARCH = "gfx950"
 # packed fp32 instructions are switched off for every device translation unit
 DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -48,7 +48,10 @@ def build(verbose: bool = True) -> Path:
     OUT_DIR.mkdir(exist_ok=True)
     srcs = [CSRC / s for s in SOURCES if (CSRC / s).exists()]
     objs = [OUT_DIR / (s.stem + ".o") for s in srcs]
-    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+    # the slowest files first: the weight-only tile kernels take minutes each
+    order = sorted(range(len(srcs)), key=lambda i: not srcs[i].name.startswith("km_wo_"))
+    srcs, objs = [srcs[i] for i in order], [objs[i] for i in order]
+    with ThreadPoolExecutor(max_workers=min(os.cpu_count() or 4, 12, len(srcs))) as pool:
         list(pool.map(lambda p: _compile(*p), zip(srcs, objs)))
     link = [hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB)]
     done = subprocess.run(link, capture_output=True, text=True)

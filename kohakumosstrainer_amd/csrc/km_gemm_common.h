@@ -127,6 +127,12 @@ __device__ __forceinline__ uint32_t hidden_load_b32(const v4i& rsrc, int voffset
   return v;
 }
 
+__device__ __forceinline__ int fresh_thread_index() {
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
+  return tid;
+}
+
 // Epilogue of a 2 x 2 wavefront grid over a BM x BN tile of 16x16 MFMA tiles whose rows are
 // output columns: lane (r16 = lane%16, g = lane/16) of tile (t, j) holds
 // C[m0+wm+j*16+r16][n0+wn+t*16+4g .. +3]. Computes acc * post * row_scale[m] * col_scale[n] +
@@ -143,8 +149,12 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
                                            const float* __restrict__ col_scale, const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N,
                                            int m0, int n0, uint8_t* buf0, uint8_t* buf1, uint8_t* buf2, uint8_t* buf3) {
   constexpr int WTM = BM / 2, WTN = BN / 2, TM = WTM / 16, TN = WTN / 16;
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) & 3;
+  // The thread index is taken afresh and made opaque: lane-derived values of the main loop must
+  // not stay live into the epilogue, where every accumulator is read out and registers run short
+  // (a value that is spilled here would be reloaded at each of its uses inside the loop).
+  const int tid = fresh_thread_index();
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6) & 3;
   const int wm = (wave >> 1) * WTM, wn = (wave & 1) * WTN;
   const int r16 = lane & 15, g = lane >> 4;
   const bool has_bias = bias != nullptr;

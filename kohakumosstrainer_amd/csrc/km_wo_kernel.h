@@ -1,0 +1,605 @@
+// The weight-only dequant-GEMM kernel template and its launchers, shared by the translation units
+// of the forward (km_wo_gemm.hip) and of the input gradient over the stored codes (km_wo_dgrad.hip).
+#pragma once
+#include <hip/hip_fp16.h>
+#include <stdio.h>
+
+#include "km_gemm_common.h"
+#include "km_wo_tiles.h"
+
+namespace km {
+
+#ifndef KM_WO_KNOCK
+#define KM_WO_KNOCK 0
+#endif
+#ifdef KM_WO_STAMPS
+__device__ unsigned long long g_wo_stamps[256];
+__device__ __forceinline__ uint64_t wo_cycles() { return __builtin_amdgcn_s_memtime(); }
+#define WO_STAMP(i) do { uint64_t now_ = wo_cycles(); st_acc[i] += now_ - st_last; st_last = now_; } while (0)
+#else
+#define WO_STAMP(i) do {} while (0)
+#endif
+constexpr int kWoStepElems = 64;  // contraction elements per step (128 B of 16-bit values)
+
+template <int DT>
+__device__ __forceinline__ void mfma16(v4f& c, const v4i& a, const v4i& b) {
+  if constexpr (DT == KM_BF16)
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  else
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
+typedef float v2f __attribute__((ext_vector_type(2)));
+
+// four e4m3 codes of one dword -> four fp32 (V_CVT_PK_F32_FP8, two codes per instruction)
+__device__ __forceinline__ void e4m3x4_to_f32(uint32_t w, float (&f)[4]) {
+  const v2f lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+  f[0] = lo.x; f[1] = lo.y; f[2] = hi.x; f[3] = hi.y;
+}
+// four e4m3 codes -> two dwords of the activation type: every e4m3 value is exact in bf16 and
+// f16, so the scaled conversion with scale 1 is the whole job (two codes per instruction)
+template <int DT>
+__device__ __forceinline__ uint2 e4m3x4_to_16(uint32_t w) {
+  if constexpr (DT == KM_BF16)
+    return make_uint2(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false)),
+                      __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true)));
+  else
+    return make_uint2(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false)),
+                      __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true)));
+}
+
+// 8 codes (two dwords) -> 8 values of the activation type (four dwords); `s` scales them in
+// fp32 before the single rounding (dgrad), or is unused (forward: the conversion is exact)
+template <int DT, int QF, bool SCALE>
+__device__ __forceinline__ uint4 widen_codes(uint2 raw, const float (&s)[8]) {
+  if constexpr (QF == KM_Q_E4M3 && !SCALE) {
+    const uint2 lo = e4m3x4_to_16<DT>(raw.x), hi = e4m3x4_to_16<DT>(raw.y);
+    return make_uint4(lo.x, lo.y, hi.x, hi.y);
+  } else {
+    float f[8];
+    if constexpr (QF == KM_Q_E4M3) {
+      float a[4], b[4];
+      e4m3x4_to_f32(raw.x, a);
+      e4m3x4_to_f32(raw.y, b);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { f[i] = a[i]; f[4 + i] = b[i]; }
+    } else {
+      const uint32_t w[2] = {raw.x, raw.y};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] = (float)(int)(int8_t)((w[i >> 2] >> (8 * (i & 3))) & 0xFFu);
+    }
+    if constexpr (SCALE) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] *= s[i];
+    }
+    return make_uint4(pack2<DT>(f[0], f[1]), pack2<DT>(f[2], f[3]), pack2<DT>(f[4], f[5]), pack2<DT>(f[6], f[7]));
+  }
+}
+
+// d[i] holds the codes (n = i, k = 0..3) of eight rows; o[j] gets the codes (k = j, n = 0..7).
+// __builtin_amdgcn_perm(hi, lo, sel): byte i of the result is byte sel[i] of {lo: 0-3, hi: 4-7}.
+__device__ __forceinline__ void transpose_8x4(const uint32_t (&d)[8], uint2 (&o)[4]) {
+  uint32_t half[2][4];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const uint32_t* r = d + 4 * h;
+    const uint32_t a01 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u), b01 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602u);
+    const uint32_t a23 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400u), b23 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602u);
+    half[h][0] = __builtin_amdgcn_perm(a23, a01, 0x05040100u);
+    half[h][1] = __builtin_amdgcn_perm(a23, a01, 0x07060302u);
+    half[h][2] = __builtin_amdgcn_perm(b23, b01, 0x05040100u);
+    half[h][3] = __builtin_amdgcn_perm(b23, b01, 0x07060302u);
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) o[j] = make_uint2(half[0][j], half[1][j]);
+}
+
+// Epilogue of the input-gradient kernel that reads q as stored. Row 16 t + r of a wavefront's B
+// slab holds column 64 b + 4 r + j of the wavefront's WTN columns, t = j Q + b, Q = WTN / 64: lane
+// (r16, g) holds, for every b, the sixteen consecutive columns 64 b + 16 g .. + 15 of output row
+// r16, element v of tile j Q + b being column 64 b + 16 g + 4 v + j. Interior tiles go through
+// the same LDS staging as store_tile (8-byte LDS writes, 16-byte reads along rows, full-line
+// global stores); edge tiles store four columns at a time (NO % 4 == 0 here). No scale, no bias.
+template <int BM, int BN, int OUT>
+__device__ __forceinline__ void store_tile_by_fours(v4f (&acc)[BN / 32][BM / 32], uint16_t* __restrict__ C, int M, int NO, int m0,
+                                                    int n0, uint8_t* buf0, uint8_t* buf1, uint8_t* buf2, uint8_t* buf3) {
+  constexpr int WTM = BM / 2, WTN = BN / 2, TM = WTM / 16, Q = WTN / 64;
+  static_assert(BN / 32 == 4 * Q, "four column residues per 64 columns");
+  const int tid = fresh_thread_index();  // see store_tile
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6) & 3;
+  const int wm = (wave >> 1) * WTM, wn = (wave & 1) * WTN;
+  const int r16 = lane & 15, g = lane >> 4;
+  auto four = [&](int b, int j, int v) __attribute__((always_inline)) {
+    return make_uint2(pack2<OUT>(acc[b][j][v], acc[Q + b][j][v]), pack2<OUT>(acc[2 * Q + b][j][v], acc[3 * Q + b][j][v]));
+  };
+  if (m0 + BM <= M && n0 + BN <= NO && (NO & 7) == 0) {
+    constexpr int RP = WTN * 2 + 16;
+    constexpr int kMinBuf = (BM < BN ? BM : BN) * 128;
+    constexpr int HM0 = TM < 4 ? TM : 4;
+    constexpr int HM = HM0 * 16 * RP <= kMinBuf ? HM0 : (HM0 / 2) * 16 * RP <= kMinBuf ? HM0 / 2 : 1;
+    constexpr int LPR = WTN * 2 / 16;  // lanes per row on the read side
+    constexpr int RPI = 64 / LPR;      // rows per read instruction
+    static_assert(HM * 16 * RP <= kMinBuf, "epilogue staging: one buffer per wavefront");
+    __syncthreads();  // every wavefront is done reading fragments
+    uint8_t* region = wave == 0 ? buf0 : wave == 1 ? buf1 : wave == 2 ? buf2 : buf3;
+    uint8_t* out_base = reinterpret_cast<uint8_t*>(C) + ((size_t)(m0 + wm) * NO + n0 + wn) * 2;
+    const int rd_row = lane / LPR, rd_col = (lane % LPR) * 16;
+    static_for<TM / HM>([&](auto p_tag) __attribute__((always_inline)) {
+      constexpr int pass = decltype(p_tag)::value;
+      static_for<HM>([&](auto j_tag) __attribute__((always_inline)) {
+        constexpr int jj = decltype(j_tag)::value;
+        constexpr int j = pass * HM + jj;
+#pragma unroll
+        for (int b = 0; b < Q; ++b)
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            *reinterpret_cast<uint2*>(region + (jj * 16 + r16) * RP + (64 * b + 16 * g + 4 * v) * 2) = four(b, j, v);
+      });
+      // only this wavefront touches its region: LDS operations of one wavefront stay in order
+      static_for<HM * 16 / RPI>([&](auto i_tag) __attribute__((always_inline)) {
+        constexpr int i = decltype(i_tag)::value;
+        const int row = i * RPI + rd_row;  // within the pass
+        const uint4 val = *reinterpret_cast<const uint4*>(region + row * RP + rd_col);
+        __builtin_nontemporal_store(__builtin_bit_cast(v4i, val), reinterpret_cast<v4i*>(out_base + (size_t)(pass * HM * 16 + row) * NO * 2 + rd_col));
+      });
+    });
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < TM; ++j) {
+    const int m = m0 + wm + j * 16 + r16;
+#pragma unroll
+    for (int b = 0; b < Q; ++b)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int col = n0 + wn + 64 * b + 16 * g + 4 * v;
+        if (m < M && col < NO) *reinterpret_cast<uint2*>(C + (size_t)m * NO + col) = four(b, j, v);
+      }
+  }
+}
+
+// two codes (byte pair `pair` of word w) -> one dword of two values of the activation type, each
+// scaled in fp32 before its single rounding when SCALE is set
+template <int DT, int QF, bool SCALE>
+__device__ __forceinline__ uint32_t widen_pair(uint32_t w, int pair, float s0, float s1) {
+  if constexpr (QF == KM_Q_E4M3 && !SCALE) {
+    if constexpr (DT == KM_BF16)
+      return pair ? __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true))
+                  : __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));
+    else
+      return pair ? __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true))
+                  : __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false));
+  } else {
+    float f0, f1;
+    if constexpr (QF == KM_Q_E4M3) {
+      const v2f v = pair ? __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true) : __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+      f0 = v.x;
+      f1 = v.y;
+    } else {
+      f0 = (float)(int)(int8_t)((w >> (16 * pair)) & 0xFFu);
+      f1 = (float)(int)(int8_t)((w >> (16 * pair + 8)) & 0xFFu);
+    }
+    if constexpr (SCALE) {
+      f0 *= s0;
+      f1 *= s1;
+    }
+    return pack2<DT>(f0, f1);
+  }
+}
+
+// The 8 x 4 byte transposition in single instructions. Stage one, p = 4 h + i: rows 4h .. 4h+3 of
+// d, i = 0: columns 0,1 of rows 0,1; 1: columns 2,3 of rows 0,1; 2, 3: the same of rows 2,3.
+__device__ __forceinline__ uint32_t transpose_stage1(const uint32_t (&d)[8], int p) {
+  const uint32_t* r = d + 4 * (p >> 2) + 2 * ((p >> 1) & 1);
+  return __builtin_amdgcn_perm(r[1], r[0], (p & 1) ? 0x07030602u : 0x05010400u);
+}
+// Stage two, p = 4 h + j: column j of rows 4h .. 4h+3 from the stage-one words t[4h .. 4h+3]
+__device__ __forceinline__ uint32_t transpose_stage2(const uint32_t (&t)[8], int p) {
+  const uint32_t* r = t + 4 * (p >> 2);
+  const int j = p & 3;
+  // columns 0,1 come from words 0 (rows 0,1) and 2 (rows 2,3); columns 2,3 from words 1 and 3
+  return __builtin_amdgcn_perm(r[2 + (j >> 1)], r[j >> 1], (j & 1) ? 0x07060302u : 0x05040100u);
+}
+
+// how the codes are laid out and scaled
+enum { kWoFwd = 0, kWoDgradT = 1, kWoDgradN = 2 };
+// kWoFwd     codes [NO, KC]; scale fp32 [NO] applied with the bias in the epilogue
+// kWoDgradT  codes [NO, KC] (a transposed copy of q); scale fp32 [KC] applied before the rounding
+// kWoDgradN  codes [KC, NO] (q as stored); scale(n, k) by SK, applied before the rounding
+
+// LDS layout of a 32-deep slab: a row is 64 bytes (four 16-byte chunks of eight 16-bit values),
+// sixteen rows fill 1 KiB. Rows r and r+4 of a 16-row block differ in the 256-byte line, rows that
+// differ in r % 4 in the 64-byte quarter of it, and the chunk index is XORed with (r / 4) % 4: the
+// 16 lanes (16 rows, one chunk) of an MFMA fragment read hit 16 different 16-byte slots modulo 256
+// bytes, and so do 16 lanes that write four chunks of four consecutive rows.
+__device__ __forceinline__ int slab32_offset(int row, int chunk) {
+  return ((row >> 4) << 10) + (((row >> 2) & 3) << 8) + ((row & 3) << 6) + ((chunk ^ ((row >> 2) & 3)) << 4);
+}
+
+// In-loop forms without the wait states for a vector-ALU-written SGPR: inside the K loop every SGPR
+// these read is loop invariant or written by the scalar ALU (m0 still needs its one wait state).
+__device__ __forceinline__ void loop_dma_b128(const v4i& rsrc, uint32_t lds_addr, int voffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voffset), "s"(rsrc) : "memory", "m0");
+}
+__device__ __forceinline__ uint64_t loop_load_b64(const v4i& rsrc, int voffset) {
+  uint64_t v;
+  asm volatile("buffer_load_dwordx2 %0, %1, %2, 0 offen" : "=v"(v) : "v"(voffset), "s"(rsrc) : "memory");
+  return v;
+}
+__device__ __forceinline__ uint32_t loop_load_b32(const v4i& rsrc, int voffset) {
+  uint32_t v;
+  asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "=v"(v) : "v"(voffset), "s"(rsrc) : "memory");
+  return v;
+}
+__device__ __forceinline__ uint32_t loop_load_u8(const v4i& rsrc, int voffset) {
+  uint32_t v;
+  asm volatile("buffer_load_ubyte %0, %1, %2, 0 offen" : "=v"(v) : "v"(voffset), "s"(rsrc) : "memory");
+  return v;
+}
+__device__ __forceinline__ uint32_t hidden_load_u8(const v4i& rsrc, int voffset) {
+  uint32_t v;
+  asm volatile("s_nop 4\n\tbuffer_load_ubyte %0, %1, %2, 0 offen" : "=v"(v) : "v"(voffset), "s"(rsrc) : "memory");
+  return v;
+}
+
+template <int BM, int BN, int DT, int QF, int MODE, int SK>
+__global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict__ A, const uint8_t* __restrict__ Q,
+                                                      const void* __restrict__ scale_ptr, int scale_ld,
+                                                      const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int NO,
+                                                      int KC) {
+  constexpr int WTM = BM / 2, WTN = BN / 2;
+  constexpr int TM = WTM / 16, TN = WTN / 16;
+  constexpr int STAGES = 4;
+  constexpr int A_STAGE = BM * 64, B_STAGE = BN * 64;  // bytes of one 32-deep slab
+  constexpr int A_LD = BM / 64;                        // direct-to-LDS passes per step: 16 rows per wavefront and pass
+  constexpr bool NAT = MODE == kWoDgradN;
+  constexpr bool PRESCALE = MODE != kWoFwd;
+  constexpr int UNITS = NAT ? 4 : BN / 64;             // 16-byte LDS writes per thread and step
+  constexpr int NQ = NAT ? 8 : UNITS;                  // code loads per thread and step
+  constexpr int NS = !NAT ? 0 : SK == KM_WSCALE_E8M0 ? 8 : SK == KM_WSCALE_BLOCKS ? 1 : 0;  // scale loads through the vector path
+  constexpr int NV = A_LD + NQ + NS;                   // vector-memory loads issued per step, counted by hand below
+  static_assert(!NAT || BN == 256 || BN == 128, "the transposing load covers 256 or 128 columns");
+  static_assert(NV < 48, "vmcnt holds 6 bits");
+  __shared__ __attribute__((aligned(1024))) uint8_t a_ring[STAGES * A_STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t b_ring[STAGES * B_STAGE];
+
+  int tile_m, tile_n;
+  tile_of(blockIdx.x, (M + BM - 1) / BM, (NO + BN - 1) / BN, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = (wave >> 1) * WTM, wn = (wave & 1) * WTN;
+  const int r16 = lane & 15, g = lane >> 4;
+  // steps of 32 contraction elements, in rounds of four (the ring's stages and the two register
+  // sets are compile-time positions of a round): a padded step multiplies slabs of zeros
+  const int steps = ((KC + 31) / 32 + 3) & ~3;
+  constexpr int kOob = 0x7FFFFFFF;  // an offset past every buffer: the load returns 0
+
+  const v4i a_rsrc = raw_rsrc(A + (size_t)m0 * KC, (uint32_t)min((int64_t)(M - m0) * KC * 2, (int64_t)0x7FFFFFFF));
+  // K-contiguous codes: the tile's rows start at n0; codes as stored: its columns start at n0
+  const int64_t q_skip = NAT ? (int64_t)n0 : (int64_t)n0 * KC;
+  const v4i q_rsrc = raw_rsrc(Q + q_skip, (uint32_t)min((int64_t)NO * KC - q_skip, (int64_t)0x7FFFFFFF));
+
+  // direct-to-LDS A pass: lane L lands in 16-byte slot L of its wavefront's 1 KiB block, which is
+  // (row 4 (L / 16) + (L % 16) / 4, chunk (L % 4) ^ (L / 16)) of the block in the slab layout
+  const int dma_row = wave * 16 + ((lane >> 4) << 2) + ((lane & 15) >> 2);
+  const int dma_chunk = (lane & 3) ^ (lane >> 4);
+  // K-contiguous codes: four lanes cover the 32 codes of a row, a wavefront 16 rows, a unit 64 rows
+  const int q_row = wave * 16 + (lane >> 2), q_chunk = lane & 3;
+  // codes as stored: LPR lanes cover the BN columns of one row n with a dword each (the other lanes
+  // of a 128-column tile load nothing and write nothing); wavefront w owns rows n = 8 w .. 8 w + 7
+  // of the step's 32, which become chunk w of the slab rows
+  constexpr int LPR = BN / 4;
+  const bool nat_live = lane < LPR;
+  const int col4 = lane % LPR;                               // columns 4 col4 .. 4 col4 + 3 of the tile
+  const int half_w = col4 / (LPR / 2), col_l = col4 % (LPR / 2);
+  const int nat_row0 = half_w * WTN + col_l;                 // slab row of column j: nat_row0 + j * (WTN / 4)
+
+  const int a_frag = lds_offset(a_ring) + slab32_offset(wm + r16, g);  // + j KiB + stage
+  const int b_frag = lds_offset(b_ring) + slab32_offset(wn + r16, g);  // + t KiB + stage
+
+  v4f acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  // codes and scales in flight, set s & 1 for slab s
+  uint32_t raw[2][NAT ? 8 : 2 * UNITS];
+  float sc[2][8];
+  uint32_t sraw[2][NS ? NS : 1];
+#pragma unroll
+  for (int b = 0; b < 2; ++b)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sc[b][i] = 1.f;
+
+  v4i scale_rsrc = v4i{0, 0, 0, 0};
+  if constexpr (NS > 0) {
+    const int64_t bytes = SK == KM_WSCALE_E8M0 ? (int64_t)KC * scale_ld : (int64_t)((KC + 127) >> 7) * scale_ld * 4;
+    scale_rsrc = raw_rsrc(scale_ptr, (uint32_t)min(bytes, (int64_t)0x7FFFFFFF));
+  }
+
+  auto opaque = [](int v) __attribute__((always_inline)) {
+    asm volatile("" : "+v"(v));
+    return v;
+  };
+  // Columns past KC become out-of-range offsets (whole 8-element chunks, KC % 8 == 0), rows past the
+  // end are out of range by themselves: both read as zeros. One per-lane offset per slab, made
+  // opaque so that the optimizer does not carry an induction register per pass; a pass adds a
+  // uniform row stride (kOob plus a stride stays out of range: the hardware compares unsigned).
+  auto a_offset = [&](int s) __attribute__((always_inline)) {
+    const int col = s * 32 + dma_chunk * 8;
+    return opaque(col < KC ? (dma_row * KC + col) * 2 : kOob);
+  };
+  auto dma_a_pass = [&](int stage, int a_off, int i) __attribute__((always_inline)) {
+    loop_dma_b128(a_rsrc, lds_offset(a_ring) + stage * A_STAGE + (i * 4 + wave) * 1024, a_off + i * (64 * 2) * KC);
+  };
+  auto q_offset = [&](int s) __attribute__((always_inline)) {
+    if constexpr (!NAT) {
+      const int col = s * 32 + q_chunk * 8;
+      return opaque(col < KC ? q_row * KC + col : kOob);
+    } else {
+      // rows n .. n + 7 of q, this thread's four columns; the group is whole (KC % 8 == 0)
+      const int n = s * 32 + 8 * wave;
+      return opaque(n < KC && nat_live ? n * NO + 4 * col4 : kOob);
+    }
+  };
+  // piece i of the code loads of a slab into register set `set`
+  auto load_code_piece = [&](int set, int q_off, int i) __attribute__((always_inline)) {
+    if constexpr (!NAT) {
+      const uint64_t v = loop_load_b64(q_rsrc, q_off + i * 64 * KC);
+      raw[set][2 * i] = (uint32_t)v;
+      raw[set][2 * i + 1] = (uint32_t)(v >> 32);
+    } else {
+      raw[set][i] = loop_load_b32(q_rsrc, q_off + i * NO);
+    }
+  };
+  // Scales of slab s. Rows and columns past the end are clamped: their codes are zeros or belong
+  // to outputs that are never stored, the scale only has to come from valid memory.
+  auto scale_offset = [&](int s) __attribute__((always_inline)) {
+    if constexpr (NS == 0) return 0;
+    else {
+      const int n = min(s * 32 + 8 * wave, KC - 8);
+      const int k = min(n0 + 4 * col4, NO - 1);  // this thread's first output column (a column of q)
+      if constexpr (SK == KM_WSCALE_E8M0) return opaque(n * scale_ld + (k >> 5));
+      else return opaque(((n >> 7) * scale_ld + (k >> 7)) * 4);  // n .. n + 7 share a block
+    }
+  };
+  auto load_scale_piece = [&](int set, int s_off, int i) __attribute__((always_inline)) {
+    if constexpr (SK == KM_WSCALE_E8M0) sraw[set][i] = loop_load_u8(scale_rsrc, s_off + i * scale_ld);
+    else sraw[set][0] = loop_load_b32(scale_rsrc, s_off);
+  };
+  // scales that do not go through the counted vector loads: per contraction column of a transposed
+  // copy (two 16-byte loads), per row of q as stored (wavefront-uniform: scalar loads)
+  auto load_scalar_scales = [&](int set, int s) __attribute__((always_inline)) {
+    if constexpr (MODE == kWoDgradT) {
+      const float* scale = static_cast<const float*>(scale_ptr);
+      const int col = min(s * 32 + q_chunk * 8, KC - 8);  // whole chunks: KC % 8 == 0
+      const float4 lo = *reinterpret_cast<const float4*>(scale + col), hi = *reinterpret_cast<const float4*>(scale + col + 4);
+      sc[set][0] = lo.x; sc[set][1] = lo.y; sc[set][2] = lo.z; sc[set][3] = lo.w;
+      sc[set][4] = hi.x; sc[set][5] = hi.y; sc[set][6] = hi.z; sc[set][7] = hi.w;
+    } else if constexpr (NAT && SK == KM_WSCALE_ROWS) {
+      const float* scale = static_cast<const float*>(scale_ptr);
+      const int n = min(s * 32 + 8 * wave, KC - 8);  // wavefront-uniform
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sc[set][i] = scale[(size_t)(n + i) * scale_ld];
+    }
+  };
+  auto load_slab = [&](int set, int s) __attribute__((always_inline)) {
+    load_scalar_scales(set, s);
+    const int q_off = q_offset(s), s_off = scale_offset(s);
+#pragma unroll
+    for (int i = 0; i < NS; ++i) load_scale_piece(set, s_off, i);
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) load_code_piece(set, q_off, i);
+  };
+  auto dma_a = [&](int stage, int s) __attribute__((always_inline)) {
+    const int a_off = a_offset(s);
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i) dma_a_pass(stage, a_off, i);
+  };
+  // The widen-and-store work of a slab in single-instruction pieces, so that each can ride behind
+  // one MFMA. Codes as stored: 8 + 8 byte permutes turn the eight dwords (n, 4 k) into four
+  // (k, 8 n) runs `tq`. Then dword d of unit c (two values of the activation type) comes from one
+  // byte pair, and unit c (four dwords) is one 16-byte LDS write.
+  uint32_t t1[8], tq[8], w16[UNITS][4];
+  auto transpose_piece = [&](int set, int p) __attribute__((always_inline)) {  // p < 16
+    if constexpr (NAT) {
+      if (p < 8) t1[p] = transpose_stage1(raw[set], p);
+      else tq[p - 8] = transpose_stage2(t1, p - 8);  // tq[4 h + j]: rows 4h .. 4h+3 of column j
+    }
+  };
+  auto widen_piece = [&](int set, int c, int d) __attribute__((always_inline)) {
+    if constexpr (!NAT) {
+      w16[c][d] = widen_pair<DT, QF, PRESCALE>(raw[set][2 * c + (d >> 1)], d & 1, sc[set][2 * d], sc[set][2 * d + 1]);
+    } else {
+      float s0, s1;
+      if constexpr (SK == KM_WSCALE_ROWS) { s0 = sc[set][2 * d]; s1 = sc[set][2 * d + 1]; }
+      else if constexpr (SK == KM_WSCALE_E8M0) { s0 = bits_f32(sraw[set][2 * d] << 23); s1 = bits_f32(sraw[set][2 * d + 1] << 23); }
+      else { s0 = s1 = bits_f32(sraw[set][0]); }
+      w16[c][d] = widen_pair<DT, QF, true>(tq[4 * (d >> 1) + c], d & 1, s0, s1);  // column c, rows 2d, 2d+1
+    }
+  };
+  auto store_unit = [&](int stage, int c) __attribute__((always_inline)) {
+    uint8_t* slab = b_ring + stage * B_STAGE;
+    const uint4 v = make_uint4(w16[c][0], w16[c][1], w16[c][2], w16[c][3]);
+    if constexpr (!NAT) *reinterpret_cast<uint4*>(slab + slab32_offset(q_row + c * 64, q_chunk)) = v;
+    else if (nat_live) *reinterpret_cast<uint4*>(slab + slab32_offset(nat_row0 + c * (WTN / 4), wave)) = v;
+  };
+  auto commit_all = [&](int set, int stage) __attribute__((always_inline)) {
+#pragma unroll
+    for (int p = 0; p < 16; ++p) transpose_piece(set, p);
+#pragma unroll
+    for (int c = 0; c < UNITS; ++c) {
+#pragma unroll
+      for (int d = 0; d < 4; ++d) widen_piece(set, c, d);
+      store_unit(stage, c);
+    }
+  };
+
+  // MFMA operands of the current step and of the next, set s & 1 for step s
+  v4i xf[2][TM], wf[2][TN];
+  typedef __attribute__((address_space(3))) const v4i* lds_v4i_cptr;
+  auto read_fragment = [&](int set, int stage, int r) __attribute__((always_inline)) {
+    // r < TM: A fragment r; else B fragment r - TM
+    if (r < TM) xf[set][r] = *(lds_v4i_cptr)(uint32_t)(a_frag + stage * A_STAGE + r * 1024);
+    else wf[set][r - TM] = *(lds_v4i_cptr)(uint32_t)(b_frag + stage * B_STAGE + (r - TM) * 1024);
+  };
+
+  // Step s (position u = s % 4 of its round) multiplies slab s out of registers that were filled
+  // during step s-1, and behind its MFMAs
+  //   starts the A loads of slab s+3 (direct to LDS, stage (u+3) % 4),
+  //   reads the fragments of slab s+1 (complete since the barrier of step s-1) into the other set,
+  //   widens the codes of slab s+2 (requested in step s-2, landed by the wait of step s-1) into stage (u+2) % 4,
+  //   requests the codes of slab s+4 into the registers just freed.
+  // The wait at its end lets this step's own NV loads stay in flight and nothing older: the A loads
+  // of slab s+2 (issued in step s-1) have landed, and with the barrier slab s+2 is complete.
+  // A 16 x 16 x 32 MFMA keeps the matrix pipe busy for 16 cycles and the wavefront can issue for
+  // 12 of them: the other work of a step is cut into pieces of one or two instructions, one piece
+  // behind each MFMA, and a scheduling barrier after every such slot keeps it there. Work that is
+  // clumped between groups of MFMAs leaves the matrix pipe idle while it issues (measured: 1640
+  // cycles per step against 1060 for the MFMAs alone).
+  constexpr int S = TN * TM;  // MFMA slots of a step
+  constexpr int NR = TM + TN;
+  constexpr int NL = NS + NQ;  // scale and code loads
+  auto at = [](int i, int n, int lo, int hi) constexpr { return lo + (i * (hi - lo)) / n; };
+#ifdef KM_WO_STAMPS
+  uint64_t st_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  uint64_t st_last = 0;
+#endif
+  int next_a_off = a_offset(3), next_q_off = q_offset(4), next_s_off = scale_offset(4);
+  auto step = [&](auto u_tag, int s) __attribute__((always_inline)) {
+    constexpr int u = decltype(u_tag)::value;
+    constexpr int par = u & 1;
+    // this step's load offsets were computed behind MFMAs of the step before
+    const int a_off = next_a_off, q_off = next_q_off, s_off = next_s_off;
+    static_for<S>([&](auto q_tag) __attribute__((always_inline)) {
+      constexpr int q = decltype(q_tag)::value;
+      constexpr int t = q / TM, j = q % TM;
+      if constexpr (!(KM_WO_KNOCK & 1)) mfma16<DT>(acc[t][j], wf[par][t], xf[par][j]);
+      else asm volatile("" :: "v"(wf[par][t]), "v"(xf[par][j]));
+      static_for<NR>([&](auto r_tag) __attribute__((always_inline)) {
+        constexpr int r = decltype(r_tag)::value;
+        if constexpr (q == at(r, NR, 0, S / 2) && !(KM_WO_KNOCK & 16)) read_fragment(par ^ 1, (u + 1) & 3, r);
+      });
+      static_for<A_LD>([&](auto i_tag) __attribute__((always_inline)) {
+        constexpr int i = decltype(i_tag)::value;
+        if constexpr (q == at(i, A_LD, 0, S / 2) && !(KM_WO_KNOCK & 8)) dma_a_pass((u + 3) & 3, a_off, i);
+      });
+      if constexpr (!(KM_WO_KNOCK & 2)) {
+        static_for<16>([&](auto p_tag) __attribute__((always_inline)) {
+          constexpr int pp = decltype(p_tag)::value;
+          if constexpr (NAT && q == at(pp, 16, S / 4, S / 2)) transpose_piece(par, pp);
+        });
+        static_for<4 * UNITS>([&](auto p_tag) __attribute__((always_inline)) {
+          constexpr int pp = decltype(p_tag)::value;
+          if constexpr (q == at(pp, 4 * UNITS, S / 2, 3 * S / 4)) widen_piece(par, pp / 4, pp % 4);
+          if constexpr (pp % 4 == 3 && q == at(pp, 4 * UNITS, S / 2, 3 * S / 4) + 1) store_unit((u + 2) & 3, pp / 4);
+        });
+      }
+      if constexpr (!(KM_WO_KNOCK & 4)) {
+        static_for<NL>([&](auto l_tag) __attribute__((always_inline)) {
+          constexpr int l = decltype(l_tag)::value;
+          if constexpr (q == at(l, NL, 3 * S / 4 + 1, S)) {
+            if constexpr (l < NS) load_scale_piece(par, s_off, l);
+            else load_code_piece(par, q_off, l - NS);
+          }
+        });
+        if constexpr (q == 3 * S / 4 + 1) load_scalar_scales(par, s + 4);
+      }
+      // the offsets of the next step's loads, a few instructions each
+      if constexpr (q == at(0, 3, S / 2, S)) next_a_off = a_offset(s + 4);
+      if constexpr (q == at(1, 3, S / 2, S)) next_q_off = q_offset(s + 5);
+      if constexpr (q == at(2, 3, S / 2, S) && NS > 0) next_s_off = scale_offset(s + 5);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    WO_STAMP(0);
+    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0((KM_WO_KNOCK & 12) ? 0 : NV));
+    WO_STAMP(1);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    WO_STAMP(2);
+  };
+
+  // prologue: slabs 0 and 1 complete, the A loads of slab 2 done, the codes of slabs 2 and 3 in
+  // registers, the fragments of slab 0 in set 0
+  dma_a(0, 0);
+  dma_a(1, 1);
+  dma_a(2, 2);
+  load_slab(0, 0);
+  load_slab(1, 1);
+  // The optimizer takes the result of a load statement for ready where the statement stands: nothing
+  // that reads it may move above the wait (in the steps every slot ends in a scheduling barrier).
+  __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+  __builtin_amdgcn_sched_barrier(0);
+  commit_all(0, 0);
+  commit_all(1, 1);
+  __builtin_amdgcn_sched_barrier(0);
+  load_slab(0, 2);
+  load_slab(1, 3);
+  __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+  __builtin_amdgcn_sched_barrier(0);
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < NR; ++r) read_fragment(0, 0, r);
+  __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+  __builtin_amdgcn_sched_barrier(0);
+#ifdef KM_WO_STAMPS
+  st_last = wo_cycles();
+#endif
+
+  for (int s = 0; s < steps; s += 4) {
+    step(std::integral_constant<int, 0>{}, s);
+    step(std::integral_constant<int, 1>{}, s + 1);
+    step(std::integral_constant<int, 2>{}, s + 2);
+    step(std::integral_constant<int, 3>{}, s + 3);
+  }
+  WO_STAMP(4);
+  // the loads of the padded slabs still in flight write LDS: let them land before the epilogue stages rows there
+  __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+
+  // the epilogue stages rows through LDS: half a ring per wavefront
+  constexpr int kQuarter = (BM < BN ? BM : BN) * 128;
+  static_assert(STAGES * A_STAGE / 2 >= kQuarter && STAGES * B_STAGE / 2 >= kQuarter, "staging room");
+  uint8_t* bufs[4] = {a_ring, a_ring + STAGES * A_STAGE / 2, b_ring, b_ring + STAGES * B_STAGE / 2};
+  if constexpr (KM_WO_KNOCK & 32) { if (acc[0][0][0] == 123.f) C[0] = 1; }
+  else if constexpr (MODE == kWoFwd)
+    store_tile<BM, BN, DT, 1>(acc, 1.0f, nullptr, static_cast<const float*>(scale_ptr), bias, C, M, NO, m0, n0, bufs[0], bufs[1], bufs[2], bufs[3]);
+  else if constexpr (MODE == kWoDgradT)
+    store_tile<BM, BN, DT, 0>(acc, 1.0f, nullptr, nullptr, nullptr, C, M, NO, m0, n0, bufs[0], bufs[1], bufs[2], bufs[3]);
+  else
+    store_tile_by_fours<BM, BN, DT>(acc, C, M, NO, m0, n0, bufs[0], bufs[1], bufs[2], bufs[3]);
+#ifdef KM_WO_STAMPS
+  WO_STAMP(5);
+  if (blockIdx.x < 8 && lane == 0)
+    for (int i = 0; i < 8; ++i) g_wo_stamps[(blockIdx.x * 4 + wave) * 8 + i] = st_acc[i];
+#endif
+}
+
+template <int BM, int BN, int DT, int QF, int MODE, int SK>
+inline int launch_wo(const void* a, const void* q, const void* scale, int scale_ld, const void* bias, void* c, int M, int NO,
+                     int KC, hipStream_t st) {
+  const int tiles = ((M + BM - 1) / BM) * ((NO + BN - 1) / BN);
+  hipLaunchKernelGGL((wo_gemm_kernel<BM, BN, DT, QF, MODE, SK>), dim3(tiles), dim3(256), 0, st, (const uint16_t*)a,
+                     (const uint8_t*)q, scale, scale_ld, (const uint16_t*)bias, (uint16_t*)c, M, NO, KC);
+  return km_check_launch("km_wo_gemm");
+}
+
+template <int DT, int QF, int MODE, int SK>
+inline int launch_config(int config, const void* a, const void* q, const void* scale, int scale_ld, const void* bias, void* c,
+                         int M, int NO, int KC, hipStream_t st) {
+  switch (config) {
+    case 0: return launch_wo<256, 256, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st);
+    case 1: return launch_wo<128, 256, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st);
+    case 2: return launch_wo<256, 128, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st);
+    case 3: return launch_wo<128, 128, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st);
+    case 4: return launch_wo<64, 128, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st);
+  }
+  return km_fail(KM_ERR_ARG, "km_wo_gemm: unknown config");
+}
+
+}  // namespace km

@@ -1,0 +1,31 @@
+// Launchers of the tiled weight-only kernels. Each activation type and direction is its own
+// translation unit (km_wo_fwd_bf16.hip, km_wo_fwd_f16.hip, km_wo_dgrad_bf16.hip, km_wo_dgrad_f16.hip):
+// the kernels take long to compile and build side by side.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "km_internal.h"
+
+namespace km {
+
+constexpr int kNumWoConfigs = 5;  // 256x256, 128x256, 256x128, 128x128, 64x128 (rows x columns of a workgroup's tile)
+
+// y = (x @ q^T) * scale + bias over K-contiguous codes q [NO, KC]
+template <int DT>
+int wo_tiles_fwd(int q_format, int config, const void* a, const void* q, const float* scale, const void* bias, void* c, int M, int NO,
+                 int KC, hipStream_t st);
+// dx = dy @ round16(q_t^T * scale) over a transposed copy q_t [NO, KC] of the codes, scale per contraction column
+template <int DT>
+int wo_tiles_dgrad_t(int q_format, int config, const void* a, const void* q_t, const float* scale, void* c, int M, int NO, int KC,
+                     hipStream_t st);
+// dx [M, K] = dy [M, N] @ round16(q [N, K] * scale(n, k)) over the codes as stored
+template <int DT>
+int wo_tiles_dgrad_n(int q_format, int scale_kind, int config, const void* dy, const void* q, const void* scale, int scale_ld, void* dx,
+                     int M, int N, int K, hipStream_t st);
+
+// argument checks shared by the entry points
+int check_wo_args(const char* who, const void* a, const void* q, const void* scale, void* c, int64_t M, int64_t N, int64_t K,
+                  int q_format, int dtype, int config);
+
+}  // namespace km

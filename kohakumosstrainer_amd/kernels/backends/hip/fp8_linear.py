@@ -10,8 +10,9 @@ MFMA-packed scales directly, the weight's packed copy comes in `aux` or is packe
 scale per output row and one per output column on the accumulator) and `block` (per K block of
 128 the MFMA's partial sum is scaled by the row's and the 128 x 128 weight block's fp32 scales
 and added to the running sum on the vector ALU). The 16-bit input gradient of a base stored
-without a dgrad copy is `dy @ dequantize(W)`: an elementwise dequantize and a plain library
-GEMM, as in the reference's `w16` path.
+without a dgrad copy (`dy @ dequantize(W)`, the reference's `w16` path, `linear.py:152-153`) is one
+kernel too: the codes are widened, scaled and rounded in registers on their way to the 16-bit
+MFMA, for every scale layout; no 16-bit copy of the weight is ever written.
 """
 
 import torch
@@ -21,7 +22,7 @@ from kohakumosstrainer_amd.kernels import registry, tuning
 from kohakumosstrainer_amd.kernels.constraints import requires
 from kohakumosstrainer_amd.kernels.hadamard import HALF
 from kohakumosstrainer_amd.kernels.errors import BackendUnavailable
-from kohakumosstrainer_amd.kernels.fp8.formats import dequantize, packed_numel
+from kohakumosstrainer_amd.kernels.fp8.formats import packed_numel
 from kohakumosstrainer_amd.kernels.fp8.op import OPS, register_launchers
 from kohakumosstrainer_amd.kernels.tuning import pow2
 
@@ -121,9 +122,39 @@ def fwd(x, q, scale, aux, bias, recipe):
     return _run(cfg, recipe, x, q, scale, aux, bias)
 
 
+def w16_candidates(m: int) -> list[dict]:
+    """Tile configurations of the 16-bit input gradient, largest first for long M."""
+    cfgs = native.configs(native.KERNEL_WO_DGRAD)
+    fits = [c for c in cfgs if c["bm"] <= max(64, pow2(m, 32))] or cfgs
+    return sorted(fits, key=lambda c: -(c["bm"] * c["bn"]) if m >= 1024 else c["bm"])
+
+
+def _dgrad_16bit(dy, q, scale, recipe):
+    """dx = dy @ round16(q * scale) over the stored codes `q [N, K]`; `scale` in `recipe`'s layout."""
+    if recipe not in GPU_RECIPES:
+        raise BackendUnavailable("fp8_dgrad", {"hip": f"recipe {recipe!r} is not built for gfx950 yet"}, persist=False)
+    m, (n, k) = dy.shape[0], q.shape
+    key = ("w16", dy.device.index, pow2(m, 32), n, k, dy.dtype, recipe)
+    cfg = _RESOLVED.get(key)
+    if cfg is None:
+        table_key = f"w16_m{pow2(m, 32)}_n{n}_k{k}_{dy.dtype}_{recipe}"
+        cfg = tuning.select(
+            "fp8_dgrad_w16",
+            dy.device,
+            table_key,
+            lambda: w16_candidates(m),
+            lambda c: lambda: native.wo_gemm_dgrad(dy, q, scale, c["id"], recipe),
+            shortlist=4,
+            in_backward=True,
+        )
+        if tuning.decided("fp8_dgrad_w16", dy.device, table_key):
+            _RESOLVED[key] = cfg
+    return native.wo_gemm_dgrad(dy, q, scale, cfg["id"], recipe)
+
+
 def dgrad(dy, q, scale, q_t, scale_t, aux_t, recipe):
     if q_t is None:
-        return dy @ dequantize(q, scale, recipe, dy.dtype)
+        return _dgrad_16bit(dy, q, scale, recipe)
     _check_shapes("dgrad", dy, q_t, recipe)
     cfg = _select("dgrad", dy, q_t, scale_t, aux_t, None, recipe, True)
     return _run(cfg, recipe, dy, q_t, scale_t, aux_t, None)

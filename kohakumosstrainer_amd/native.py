@@ -45,6 +45,7 @@ EXPORTS = (
     "km_gemm_i8_rows",
     "km_wo_gemm_fwd",
     "km_wo_gemm_dgrad",
+    "km_wo_gemm_dgrad_w16",
     "km_wo_gemm_dgrad_static",
     "km_group_hadamard",
     "km_num_configs",
@@ -85,6 +86,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.km_gemm_i8_rows.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, p]
     lib.km_wo_gemm_fwd.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_wo_gemm_dgrad.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
+    lib.km_wo_gemm_dgrad_w16.argtypes = [p, p, p, i32, i64, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_wo_gemm_dgrad_static.argtypes = [p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_group_hadamard.argtypes = [p, i64, i64, i32, i32, p, p]
     lib.km_num_configs.argtypes = [i32]
@@ -525,8 +527,53 @@ def wo_gemm_fwd(x: Tensor, q: Tensor, scale: Tensor, bias: Tensor | None, config
     return y
 
 
-def wo_gemm_dgrad(dy: Tensor, q: Tensor, scale: Tensor, config: int = 0) -> Tensor:
-    """`dy @ round(q * scale[:, None])` -> `[M, K]` in dy's dtype."""
+WSCALE_ROWS, WSCALE_E8M0, WSCALE_BLOCKS = 0, 1, 2  # weight scale layouts of km_wo_gemm_dgrad_w16
+
+
+def wo_gemm_dgrad(dy: Tensor, q: Tensor, scale: Tensor, config: int = 0, recipe: str = "row") -> Tensor:
+    """`dy @ round(q * scale)` -> `[M, K]` in dy's dtype, over the codes `q [N, K]` as they are
+    stored (no transposed copy, no workspace). `recipe` names the scale layout: "row" fp32 `[N]`,
+    "tensor" one fp32, "mx" uint8 `[N, K/32]` biased exponents, "block" fp32 `[ceil(N/128), K/128]`
+    (the last three for e4m3 codes)."""
+    if dy.dim() != 2 or q.dim() != 2 or dy.shape[1] != q.shape[0]:
+        raise ValueError(f"dy must be [M, N] and q [N, K], got {tuple(dy.shape)} and {tuple(q.shape)}")
+    if q.dtype not in _QFORMATS:
+        raise ValueError(f"codes must be int8 or float8_e4m3fn, got {q.dtype}")
+    m, n = dy.shape
+    k = q.shape[1]
+    _on_gpu(dy, q, scale)
+    dy, q = dy.contiguous(), q.contiguous()
+    if recipe == "row":
+        kind, ld, scale = WSCALE_ROWS, 1, scale.float().reshape(-1).contiguous()
+        want = n
+    elif recipe == "tensor":
+        kind, ld, scale = WSCALE_ROWS, 0, scale.float().reshape(-1).contiguous()
+        want = 1
+    elif recipe == "mx":
+        scale = scale.contiguous()
+        if scale.dtype != torch.uint8 or scale.dim() != 2 or scale.shape[0] != n:
+            raise ValueError(f"mx scales must be uint8 [N, K/32], got {scale.dtype} {tuple(scale.shape)}")
+        kind, ld, want = WSCALE_E8M0, scale.shape[1], n * ((k + 31) // 32)
+    elif recipe == "block":
+        scale = scale.float().contiguous()
+        if scale.dim() != 2 or scale.shape[0] != (n + 127) // 128:
+            raise ValueError(f"block scales must be [ceil(N/128), K/128], got {tuple(scale.shape)}")
+        kind, ld, want = WSCALE_BLOCKS, scale.shape[1], ((n + 127) // 128) * ((k + 127) // 128)
+    else:
+        raise ValueError(f"unknown scale layout {recipe!r}")
+    if scale.numel() < want:
+        raise ValueError(f"{recipe} scales of q {tuple(q.shape)} need {want} values, got {scale.numel()}")
+    if q.dtype == torch.int8 and kind != WSCALE_ROWS:
+        raise ValueError("int8 codes take one scale per row")
+    dx = torch.empty(m, k, device=dy.device, dtype=dy.dtype)
+    with torch.cuda.device(dy.device):
+        _check(load().km_wo_gemm_dgrad_w16(dy.data_ptr(), q.data_ptr(), scale.data_ptr(), kind, ld, dx.data_ptr(), m, n, k, _QFORMATS[q.dtype], _dtype_code(dy.dtype), config, _stream(dy)))
+    return dx
+
+
+def wo_gemm_dgrad_workspace(dy: Tensor, q: Tensor, scale: Tensor, config: int = 0) -> Tensor:
+    """The same input gradient through `km_wo_gemm_dgrad`: the codes are first transposed into an
+    N * K byte workspace that this wrapper allocates."""
     dy, q, scale = _wo_operands(dy, q, scale)
     if dy.shape[1] != q.shape[0]:
         raise ValueError(f"dy is [M, {dy.shape[1]}] but q is [{q.shape[0]}, K]")

@@ -65,7 +65,7 @@ def check(got, eager, exact, dtype, what, slack=1.0):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("recipe,dgrad", [("mx", True), ("mx", False), ("tensor", True), ("row", True), ("row", False), ("block", True), ("block", False)])
+@pytest.mark.parametrize("recipe,dgrad", [("mx", True), ("mx", False), ("tensor", True), ("tensor", False), ("row", True), ("row", False), ("block", True), ("block", False)])
 def test_fp8_linear_forward_and_grads(dtype, recipe, dgrad):
     m, n, k = 300, 384, 512
     x, w, bias, dy, base = problem(m, n, k, dtype, recipe, dgrad)

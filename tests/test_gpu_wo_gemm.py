@@ -55,10 +55,84 @@ def test_forward_and_dgrad(fmt, dtype, m, n, k, with_bias):
         assert rel_l2(y.cpu(), truth) <= tol
     truth_dx = dy.double() @ w64
     eager_dx = linear.wo_dgrad(dy, q, scale)
-    for cfg in (0, n_configs() - 1):
+    first = None
+    for cfg in range(n_configs()):
         dx = native.wo_gemm_dgrad(dy.cuda(), q.cuda(), scale.cuda(), cfg)
         assert dx.shape == (m, k) and dx.dtype == dtype
         assert_no_regression(dx.cpu(), eager_dx, truth_dx, f"wo dgrad {fmt} cfg{cfg} {m}x{n}x{k}")
+        # every tile shape sums a row's products in the same order
+        first = dx if first is None else first
+        assert torch.equal(dx, first), f"cfg{cfg} differs from cfg0"
+    if n % 8 == 0:
+        # the entry point that transposes the codes into a workspace first feeds the MFMA the same operands
+        assert torch.equal(native.wo_gemm_dgrad_workspace(dy.cuda(), q.cuda(), scale.cuda(), 0), first)
+
+
+def fp8_base(n, k, recipe, seed=0):
+    """(q, scale) of a frozen fp8 compute base quantized by the oracle, plus its exact fp64 value."""
+    from oracle import formats
+
+    g = torch.Generator().manual_seed(seed)
+    w = (torch.randn(n, k, generator=g) * 0.05).to(torch.bfloat16)
+    q, scale = formats.quantize(w, recipe, "weight")
+    w64 = formats.dequantize(q, scale, recipe, torch.float64)
+    return q, scale, w64
+
+
+@pytest.mark.parametrize("recipe", ("tensor", "row", "mx", "block"))
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+@pytest.mark.parametrize("m,n,k", ((200, 256, 384), (64, 128, 128), (513, 1024, 640), (300, 384, 1152)))
+def test_input_gradient_of_an_fp8_base_without_a_transposed_copy(recipe, dtype, m, n, k):
+    """dx = dy @ dequantize(q, scale) over the codes as stored, for every scale layout of the fp8
+    compute recipes (reference `backends/triton/fp8/linear.py:152-153`): against the fp64 product
+    with the exactly dequantized weight, next to the oracle's eager result (10x rule), every tile
+    shape; the widened weight itself is read back through identity rows, bit for bit."""
+    from oracle import formats
+
+    q, scale, w64 = fp8_base(n, k, recipe)
+    g = torch.Generator().manual_seed(5)
+    dy = torch.randn(m, n, generator=g).to(dtype)
+    truth = dy.double() @ w64
+    eager = linear.fp8_dgrad(dy, q, scale, None, None, None, recipe)
+    for cfg in range(n_configs()):
+        dx = native.wo_gemm_dgrad(dy.cuda(), q.cuda(), scale.cuda(), cfg, recipe)
+        assert dx.shape == (m, k) and dx.dtype == dtype
+        assert_no_regression(dx.cpu(), eager, truth, f"w16 dgrad {recipe} cfg{cfg} {m}x{n}x{k}")
+    eye = torch.eye(n, dtype=dtype)[:256]
+    back = native.wo_gemm_dgrad(eye.cuda(), q.cuda(), scale.cuda(), 0, recipe).cpu()
+    assert torch.equal(back, formats.dequantize(q, scale, recipe, dtype)[:256])
+
+
+@pytest.mark.parametrize("fmt,recipe", (("int8", "row"), ("fp8", "row"), ("fp8", "mx")))
+@pytest.mark.parametrize("m,n,k", ((37, 100, 50), (130, 96, 66), (16, 64, 1), (5, 0, 64)))
+def test_input_gradient_shapes_off_the_vector_path(fmt, recipe, m, n, k):
+    """N not a multiple of 8, K not a multiple of 4, an empty contraction, a misaligned operand: the
+    one-thread-per-element kernel, judged by the same rule."""
+    from oracle import formats
+
+    g = torch.Generator().manual_seed(11)
+    if recipe == "mx":
+        n, k = max(n, 32), 64 if k < 32 else 96
+        w = (torch.randn(n, k, generator=g) * 0.05).to(torch.bfloat16)
+        q, scale = formats.quantize(w, "mx", "weight")
+        w64 = formats.dequantize(q, scale, "mx", torch.float64)
+        dy = torch.randn(m, n, generator=g).to(torch.bfloat16)
+        eager = linear.fp8_dgrad(dy, q, scale, None, None, None, "mx")
+        # a view one element into a buffer: the pointer is not 16-byte aligned
+        shifted = torch.empty(m * n + 1, dtype=torch.bfloat16, device="cuda")[1:].view(m, n).copy_(dy)
+        dx = native.wo_gemm_dgrad(shifted, q.cuda(), scale.cuda(), 0, "mx")
+    else:
+        w = torch.randn(n, k, generator=g) * 0.05
+        q, scale = linear.quantize_weight(w, fmt) if n else (torch.zeros(0, k, dtype=torch.int8 if fmt == "int8" else torch.float8_e4m3fn), torch.zeros(0))
+        w64 = linear.wo_exact64(q, scale)
+        dy = torch.randn(m, n, generator=g).to(torch.bfloat16)
+        eager = linear.wo_dgrad(dy, q, scale)
+        dx = native.wo_gemm_dgrad(dy.cuda(), q.cuda(), scale.cuda(), 0, "row")
+    assert dx.shape == (m, k)
+    if n == 0:
+        assert not dx.any(), "an empty contraction gives zeros"
+        return
+    assert_no_regression(dx.cpu(), eager, dy.double() @ w64, f"scalar dgrad {fmt} {recipe} {m}x{n}x{k}")
 
 
 def test_int8_forward_is_exact_product_for_small_integers():
