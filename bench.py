@@ -275,6 +275,46 @@ def other_configs(dev, reps):
     return out
 
 
+def same_node(dev, x, w, bias, reps):
+    """The vendor library on the same card and the same headline shape, the comparison the reference's
+    own benchmark prints (scripts/bench/kernel/fp8.py: bf16 F.linear and torch._scaled_mm): bf16
+    GEMM, fp8 GEMM with one scale per tensor, with one scale per row / column, and with E8M0 block
+    scales. Each in a try block: what this torch / hipBLASLt build does not offer is reported as such.
+    These are library calls timed for reference only; no product path uses them."""
+    out = {}
+    flop = 2 * x.shape[0] * x.shape[1] * w.shape[0]
+
+    def timed(name, fn, peak):
+        try:
+            fn()
+            ms = event_ms(fn, reps)
+            out[name] = {"ms": ms, "TFLOPs": flop / ms / 1e9, "frac": flop / ms / 1e9 / peak}
+        except Exception as err:  # noqa: BLE001 - reported, not swallowed
+            out[name] = {"unavailable": f"{type(err).__name__}: {str(err)[:160]}"}
+
+    timed("bf16_F_linear", lambda: torch.nn.functional.linear(x, w, bias), 2500.0)
+    e4m3 = torch.float8_e4m3fn
+    xa, wa = x.float().abs().amax(), w.float().abs().amax()
+    sx, sw = (xa / 448.0).reshape(()), (wa / 448.0).reshape(())
+    xq8, wq8 = (x.float() / sx).to(e4m3), (w.float() / sw).to(e4m3)
+    timed("fp8_scaled_mm_tensor", lambda: torch._scaled_mm(xq8, wq8.t(), scale_a=sx, scale_b=sw, bias=bias, out_dtype=torch.bfloat16), FP8_PEAK_TFLOPS)
+    sxr = (x.float().abs().amax(1, keepdim=True) / 448.0).clamp_min(1e-12)
+    swr = (w.float().abs().amax(1, keepdim=True) / 448.0).clamp_min(1e-12)
+    xqr, wqr = (x.float() / sxr).to(e4m3), (w.float() / swr).to(e4m3)
+    timed("fp8_scaled_mm_rows", lambda: torch._scaled_mm(xqr, wqr.t(), scale_a=sxr, scale_b=swr.t(), bias=bias, out_dtype=torch.bfloat16), FP8_PEAK_TFLOPS)
+    e8m0 = getattr(torch, "float8_e8m0fnu", None)
+    if e8m0 is None:
+        out["fp8_scaled_mm_mx"] = {"unavailable": "torch has no float8_e8m0fnu"}
+    else:
+        from kohakumosstrainer_amd import native
+
+        xq, xs = native.quant_mx(x)[:2]
+        wq, ws = native.quant_mx(w)[:2]
+        timed("fp8_scaled_mm_mx", lambda: torch._scaled_mm(xq, wq.t(), scale_a=xs.view(e8m0), scale_b=ws.view(e8m0), bias=bias, out_dtype=torch.bfloat16), FP8_PEAK_TFLOPS)
+    out["note"] = "vendor library GEMMs alone (no activation quantizer in the timed call), same card, same operands' shape; frac is of the same peak as this build's kernels"
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -360,7 +400,20 @@ def main():
         event_ms(f, 10)
     rows_cold_ms = event_ms(cold(lambda t: t), max(args.steps, 10))
     cols_cold_ms = event_ms(cold(lambda t: t.t()), max(args.steps, 10))
-    del ring, held
+    # what a plain device copy of the same number of bytes takes on the same ring: the ceiling a
+    # streaming kernel can reach on this card (a copy moves QUANT_BYTES / 1.5 * 2 bytes per call of
+    # bf16 in and out; scaled to the quantizer's byte count)
+    copies = [torch.empty_like(ring[0]) for _ in range(5)]
+
+    def cold_copy():
+        i = state["i"] = (state["i"] + 1) % 5
+        copies[i].copy_(ring[i])
+
+    event_ms(cold_copy, 10)
+    copy_cold_ms = event_ms(cold_copy, max(args.steps, 10))
+    copy_bytes = 2 * ring[0].numel() * 2
+    copy_GBps = copy_bytes / (copy_cold_ms * 1e-3) / 1e9
+    del ring, held, copies
     achieved = GEMM_FLOP / (gemm_ms * 1e-3) / 1e12
 
     line = {
@@ -408,11 +461,17 @@ def main():
             "cols_cold_ms": cols_cold_ms,
             "cols_cold_GBps": QUANT_BYTES / (cols_cold_ms * 1e-3) / 1e9,
             "cols_cold_frac": QUANT_BYTES / (cols_cold_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "note": "rows_/cols_: back-to-back launches on one tensor (the reference's timing method; part of it stays in the 256 MB last-level cache); *_cold_: a ring of tensors larger than that cache",
+            "copy_cold_ms": copy_cold_ms,
+            "copy_cold_GBps": copy_GBps,
+            "copy_cold_frac": copy_GBps / HBM_PEAK_GBS,
+            "rows_cold_vs_copy": (QUANT_BYTES / (rows_cold_ms * 1e-3) / 1e9) / copy_GBps,
+            "cols_cold_vs_copy": (QUANT_BYTES / (cols_cold_ms * 1e-3) / 1e9) / copy_GBps,
+            "note": "rows_/cols_: back-to-back launches on one tensor (the reference's timing method; part of it stays in the 256 MB last-level cache); *_cold_: a ring of tensors larger than that cache; copy_cold_: torch's device copy of one ring tensor (read + write), the practical HBM ceiling of a streaming kernel here",
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
         },
     }
+    line["same_node"] = same_node(dev, x, w, bias, max(args.steps // 2, 5))
     line["other_configs"] = other_configs(dev, max(args.steps // 2, 5))
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(x, wq, ws, bias)

@@ -109,6 +109,13 @@ __device__ __forceinline__ void hidden_dma_b128(const v4i& rsrc, uint32_t lds_ad
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                ::"s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
 }
+// The same load for use inside a K loop whose SGPR operands (descriptor, soffset, the LDS address) are
+// loop invariant or written by the scalar ALU: only m0 needs its one wait state. The five wait states of
+// the general form keep the matrix pipe idle once per load when it rides behind an MFMA.
+__device__ __forceinline__ void loop_dma_b128(const v4i& rsrc, uint32_t lds_addr, int voffset, int soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               ::"s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
+}
 // 4 bytes per lane to lds_addr + 4 * lane: used to pull lines into L2 ahead of their real fetch,
 // aimed at LDS bytes that a later load of the same wavefront overwrites
 __device__ __forceinline__ void hidden_touch_b32(const v4i& rsrc, uint32_t lds_addr, int voffset, int soffset) {

@@ -201,6 +201,13 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
   auto dma_b_pass = [&](uint32_t buf, int koff, int i, int beyond = 0) __attribute__((always_inline)) {
     hidden_dma_b128(b_rsrc, buf + i * 4096 + wave * 1024, ld_voff + i * pass_stride + beyond, koff);
   };
+  // inside the K loop: every SGPR these read is loop invariant or comes from the scalar ALU
+  auto loop_dma_a_pass = [&](uint32_t buf, int koff, int i) __attribute__((always_inline)) {
+    loop_dma_b128(a_rsrc, buf + i * 4096 + wave * 1024, ld_voff + i * pass_stride, koff);
+  };
+  auto loop_dma_b_pass = [&](uint32_t buf, int koff, int i, int beyond = 0) __attribute__((always_inline)) {
+    loop_dma_b128(b_rsrc, buf + i * 4096 + wave * 1024, ld_voff + i * pass_stride + beyond, koff);
+  };
   auto dma_a = [&](uint32_t buf, int ks) __attribute__((always_inline)) {
     const int koff = __builtin_amdgcn_readfirstlane(ks * kStepBytes);
 #pragma unroll
@@ -331,7 +338,7 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
             constexpr int i = decltype(i_tag)::value;
             if constexpr (q == (A1 ? i : i * kBWindow / B_LD)) {
               __builtin_amdgcn_sched_barrier(0);
-              dma_b_pass(b_fill, koff_b, i, b_beyond);
+              loop_dma_b_pass(b_fill, koff_b, i, b_beyond);
               __builtin_amdgcn_sched_barrier(0);
             }
           });
@@ -346,7 +353,7 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
                 __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
                 __syncthreads();
               }
-              dma_a_pass(a_cur, koff_a, i);
+              loop_dma_a_pass(a_cur, koff_a, i);
               __builtin_amdgcn_sched_barrier(0);
             }
           });

@@ -219,9 +219,6 @@ __device__ __forceinline__ int slab32_offset(int row, int chunk) {
 
 // In-loop forms without the wait states for a vector-ALU-written SGPR: inside the K loop every SGPR
 // these read is loop invariant or written by the scalar ALU (m0 still needs its one wait state).
-__device__ __forceinline__ void loop_dma_b128(const v4i& rsrc, uint32_t lds_addr, int voffset) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voffset), "s"(rsrc) : "memory", "m0");
-}
 __device__ __forceinline__ uint64_t loop_load_b64(const v4i& rsrc, int voffset) {
   uint64_t v;
   asm volatile("buffer_load_dwordx2 %0, %1, %2, 0 offen" : "=v"(v) : "v"(voffset), "s"(rsrc) : "memory");
@@ -333,7 +330,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
     return opaque(col < KC ? (dma_row * KC + col) * 2 : kOob);
   };
   auto dma_a_pass = [&](int stage, int a_off, int i) __attribute__((always_inline)) {
-    loop_dma_b128(a_rsrc, lds_offset(a_ring) + stage * A_STAGE + (i * 4 + wave) * 1024, a_off + i * (64 * 2) * KC);
+    loop_dma_b128(a_rsrc, lds_offset(a_ring) + stage * A_STAGE + (i * 4 + wave) * 1024, a_off + i * (64 * 2) * KC, 0);
   };
   auto q_offset = [&](int s) __attribute__((always_inline)) {
     if constexpr (!NAT) {
