@@ -17,6 +17,7 @@ from torch import Tensor
 LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libkm_kernels.so"
 E4M3 = torch.float8_e4m3fn
 KM_BF16, KM_F16 = 0, 1
+KM_OK, KM_ERR_ARG, KM_ERR_LAUNCH, KM_ERR_UNSUPPORTED = 0, -1, -2, -3  # return codes of every entry point
 KM_Q_INT8, KM_Q_E4M3 = 0, 1
 KERNEL_GEMM_MX, KERNEL_GEMM_FP8, KERNEL_WO_FWD, KERNEL_WO_DGRAD, KERNEL_GEMM_BLOCKS = 0, 1, 2, 3, 4
 ROLE_ACT, ROLE_WEIGHT = 0, 1
