@@ -22,11 +22,24 @@ _LIMIT = {"int8": 127.0, "fp8": 448.0}
 _FLOOR = 1e-12
 
 
+def _hip_rows(w: Tensor) -> bool:
+    if not (w.is_cuda and w.dtype in (torch.bfloat16, torch.float16)):
+        return False
+    from kohakumosstrainer_amd.kernels.arch import arch_of
+
+    return arch_of(w.device).name == "gfx950"
+
+
 def quantize(w: Tensor, fmt: str) -> tuple[Tensor, Tensor]:
     """Per-output-row symmetric quantizer. The scale is `max(amax, 1e-12) / limit` with the limit
     a Python number (127 for int8: codes round half to even; 448 for e4m3: one rounding of w / s)."""
     if fmt not in FORMATS:
         raise ValueError(f"quant format {fmt!r} not in {FORMATS}")
+    if w.dim() == 2 and _hip_rows(w):
+        # 16-bit weights on the card: the per-row quantizer kernels (same scale, same single rounding)
+        from kohakumosstrainer_amd import native
+
+        return native.quant_rows_i8(w.detach(), None) if fmt == "int8" else native.quant_rows(w.detach())
     v = w.detach().to(torch.float32)
     scale = v.abs().amax(dim=1).clamp_min(_FLOOR) / _LIMIT[fmt]
     ratio = v / scale.unsqueeze(1)

@@ -278,3 +278,23 @@ def test_lora_training_step_over_frozen_mxfp8_base():
     up_ref = dy.double().t() @ (x.double() @ down.double().t())
     dn_ref = (dy.double() @ up.double()).t() @ x.double()
     assert oracle_stats.rel_l2(upd.grad.cpu(), up_ref) < 1e-2 and oracle_stats.rel_l2(dn.grad.cpu(), dn_ref) < 1e-2
+
+
+@pytest.mark.parametrize("fmt", ("int8", "fp8"))
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+@pytest.mark.parametrize("n,k", ((3072, 3072), (100, 136), (7, 40)))
+def test_weight_quantizer_on_the_card_equals_the_oracle(fmt, dtype, n, k):
+    """`weights.quantize` of a 16-bit weight on the GPU runs the per-row quantizer kernels: codes
+    and scales bit for bit those of the oracle's frozen-base quantizer (reference
+    `src/kohakumoss/quant/weights.py:31-43`), an all-zero row and a row with one huge entry included."""
+    from kohakumosstrainer_amd.quant.weights import quantize
+
+    g = torch.Generator().manual_seed(n + k)
+    w = (torch.randn(n, k, generator=g) * 0.05).to(dtype)
+    w[0] = 0
+    w[1, 3] = 300.0
+    q_want, s_want = oracle_linear.quantize_weight(w, fmt)
+    q, s = quantize(w.cuda(), fmt)
+    assert q.dtype == q_want.dtype and s.dtype == torch.float32
+    assert torch.equal(s.cpu(), s_want)
+    assert torch.equal(q.cpu().view(torch.uint8), q_want.view(torch.uint8))

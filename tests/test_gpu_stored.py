@@ -53,3 +53,36 @@ def test_stored_checkpoint_runs_on_the_hip_backend(tmp_path, recipe):
     truth = linear.exact64(xq, xs, recipe) @ linear.exact64(src.up.base.q, src.up.base.scale, recipe).T + src.up.bias.double()
     assert y.dtype == torch.bfloat16 and rel_l2(y.cpu(), truth) <= 2e-3
     assert torch.isfinite(model(x.cuda())).all()
+
+
+@pytest.mark.parametrize("recipe,dgrad", (("mx", True), ("mx", False), ("row", False)))
+def test_streamed_slot_view_on_the_hip_backend(recipe, dgrad):
+    """A streamed fp8 base on the card: the slot is refilled with another layer between forward and
+    backward; output and gradients equal the resident base's bit for bit (with `dgrad` off the input
+    gradient is the 16-bit kernel over the slot's codes)."""
+    from kohakumosstrainer_amd.quant.compute import StreamedParts
+
+    registry.load_backends()
+    g = torch.Generator().manual_seed(1)
+    make = lambda: ComputeWeight.from_weight((torch.randn(384, 256, generator=g) * 0.05).to(torch.bfloat16).cuda(), recipe, dgrad)
+    layer_a, layer_b = make(), make()
+    slot = {name: t.clone() for name, t in layer_a.tensors().items()}
+
+    def fetch_a():
+        for name, t in layer_a.tensors().items():
+            slot[name].copy_(t)
+        return slot
+
+    view = StreamedParts(recipe, fetch_a, torch.bfloat16, "cuda")
+    x = torch.randn(200, 256, generator=g).to(torch.bfloat16).cuda().requires_grad_()
+    bias = torch.randn(384, generator=g).to(torch.bfloat16).cuda().requires_grad_()
+    dy = torch.randn(200, 384, generator=g).to(torch.bfloat16).cuda()
+    y = view.linear(x, bias)
+    for name, t in layer_b.tensors().items():
+        slot[name].copy_(t)
+    y.backward(dy)
+    x2, b2 = x.detach().clone().requires_grad_(), bias.detach().clone().requires_grad_()
+    y2 = layer_a.linear(x2, b2)
+    y2.backward(dy)
+    assert torch.equal(y.detach(), y2.detach())
+    assert torch.equal(x.grad, x2.grad) and torch.equal(bias.grad, b2.grad)

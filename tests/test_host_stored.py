@@ -172,3 +172,38 @@ def test_meta_initialised_model_loads_without_dense_copies(tmp_path):
     assert empty.a.weight.numel() == 0 and not any(p.is_meta for p in empty.parameters())
     x = torch.randn(3, 256)
     assert torch.equal(empty(x), m(x))
+
+
+def test_streamed_slot_linear_holds_no_slot_tensor_in_the_graph():
+    """A weight-streaming ring refills its slot between a layer's forward and backward. The
+    streamed view must fetch the parts again for the input gradient: here the slot buffers are
+    overwritten with another layer's codes right after the forward, and `fetch` copies the right
+    layer back in when asked. Gradients equal those of the resident base."""
+    from kohakumosstrainer_amd.quant.compute import ComputeWeight, StreamedParts
+
+    g = torch.Generator().manual_seed(0)
+    w_a, w_b = torch.randn(96, 128, generator=g) * 0.05, torch.randn(96, 128, generator=g) * 0.05
+    layers = {"a": ComputeWeight.from_weight(w_a, "mx", dgrad=True), "b": ComputeWeight.from_weight(w_b, "mx", dgrad=True)}
+    slot = {name: t.clone() for name, t in layers["a"].tensors().items()}
+    fetched = []
+
+    def fetch_a():
+        fetched.append(len(fetched))
+        for name, t in layers["a"].tensors().items():
+            slot[name].copy_(t)
+        return slot
+
+    view = StreamedParts("mx", fetch_a, torch.float32, "cpu")
+    x = torch.randn(10, 128, generator=g, requires_grad=True)
+    bias = torch.randn(96, generator=g, requires_grad=True)
+    y = view.linear(x, bias)
+    for name, t in layers["b"].tensors().items():  # the ring moves on to another layer
+        slot[name].copy_(t)
+    y.backward(torch.ones_like(y))
+    assert len(fetched) == 2, "one fetch per direction"
+    x2 = x.detach().clone().requires_grad_()
+    b2 = bias.detach().clone().requires_grad_()
+    layers["a"].linear(x2, b2).backward(torch.ones_like(y))
+    assert torch.equal(y.detach(), layers["a"].linear(x2, b2).detach())
+    assert torch.equal(x.grad, x2.grad) and torch.equal(bias.grad, b2.grad)
+    assert torch.equal(view.weight(torch.float32), layers["a"].weight(torch.float32))
