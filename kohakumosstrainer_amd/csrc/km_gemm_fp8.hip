@@ -420,6 +420,13 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
   // retire before the accumulators are read
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  // The compiler does not know that the opaque MFMAs' results take time and copies accumulators to
+  // vector registers wherever it likes (the loop exit included): passing every accumulator through an
+  // empty statement placed after the wait makes each later read depend on it.
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) asm volatile("" : "+a"(acc[i][j]));
   __builtin_amdgcn_sched_barrier(0);
 
   // epilogue: bias (and the per-tensor scales) on the fp32 accumulator, one rounding

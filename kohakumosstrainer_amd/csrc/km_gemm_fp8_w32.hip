@@ -397,6 +397,13 @@ __global__ __launch_bounds__(256, 1) void gemm_fp8_w32_kernel(
   // each) time to retire before the accumulators are read
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  // The compiler does not know that the opaque MFMAs' results take time and copies accumulators to
+  // vector registers wherever it likes (the loop exit included): passing every accumulator through an
+  // empty statement placed after the wait makes each later read depend on it.
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) asm volatile("" : "+a"(acc[i][j]));
   __builtin_amdgcn_sched_barrier(0);
 
   float post = 1.0f;

@@ -9,16 +9,6 @@
 
 namespace km {
 
-#ifndef KM_WO_KNOCK
-#define KM_WO_KNOCK 0
-#endif
-#ifdef KM_WO_STAMPS
-__device__ unsigned long long g_wo_stamps[256];
-__device__ __forceinline__ uint64_t wo_cycles() { return __builtin_amdgcn_s_memtime(); }
-#define WO_STAMP(i) do { uint64_t now_ = wo_cycles(); st_acc[i] += now_ - st_last; st_last = now_; } while (0)
-#else
-#define WO_STAMP(i) do {} while (0)
-#endif
 constexpr int kWoStepElems = 64;  // contraction elements per step (128 B of 16-bit values)
 
 template <int DT>
@@ -461,10 +451,8 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   constexpr int NR = TM + TN;
   constexpr int NL = NS + NQ;  // scale and code loads
   auto at = [](int i, int n, int lo, int hi) constexpr { return lo + (i * (hi - lo)) / n; };
-#ifdef KM_WO_STAMPS
-  uint64_t st_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  uint64_t st_last = 0;
-#endif
+  constexpr int L0 = 3 * S / 4;  // first slot of the code loads: the last conversion piece sits in the slot before
+  static_assert(S >= 4 && S % 4 == 0, "a step has at least four MFMA slots");
   int next_a_off = a_offset(3), next_q_off = q_offset(4), next_s_off = scale_offset(4);
   auto step = [&](auto u_tag, int s) __attribute__((always_inline)) {
     constexpr int u = decltype(u_tag)::value;
@@ -474,49 +462,41 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
     static_for<S>([&](auto q_tag) __attribute__((always_inline)) {
       constexpr int q = decltype(q_tag)::value;
       constexpr int t = q / TM, j = q % TM;
-      if constexpr (!(KM_WO_KNOCK & 1)) mfma16<DT>(acc[t][j], wf[par][t], xf[par][j]);
-      else asm volatile("" :: "v"(wf[par][t]), "v"(xf[par][j]));
+      mfma16<DT>(acc[t][j], wf[par][t], xf[par][j]);
       static_for<NR>([&](auto r_tag) __attribute__((always_inline)) {
         constexpr int r = decltype(r_tag)::value;
-        if constexpr (q == at(r, NR, 0, S / 2) && !(KM_WO_KNOCK & 16)) read_fragment(par ^ 1, (u + 1) & 3, r);
+        if constexpr (q == at(r, NR, 0, S / 2)) read_fragment(par ^ 1, (u + 1) & 3, r);
       });
       static_for<A_LD>([&](auto i_tag) __attribute__((always_inline)) {
         constexpr int i = decltype(i_tag)::value;
-        if constexpr (q == at(i, A_LD, 0, S / 2) && !(KM_WO_KNOCK & 8)) dma_a_pass((u + 3) & 3, a_off, i);
+        if constexpr (q == at(i, A_LD, 0, S / 2)) dma_a_pass((u + 3) & 3, a_off, i);
       });
-      if constexpr (!(KM_WO_KNOCK & 2)) {
-        static_for<16>([&](auto p_tag) __attribute__((always_inline)) {
-          constexpr int pp = decltype(p_tag)::value;
-          if constexpr (NAT && q == at(pp, 16, S / 4, S / 2)) transpose_piece(par, pp);
-        });
-        static_for<4 * UNITS>([&](auto p_tag) __attribute__((always_inline)) {
-          constexpr int pp = decltype(p_tag)::value;
-          if constexpr (q == at(pp, 4 * UNITS, S / 2, 3 * S / 4)) widen_piece(par, pp / 4, pp % 4);
-          if constexpr (pp % 4 == 3 && q == at(pp, 4 * UNITS, S / 2, 3 * S / 4) + 1) store_unit((u + 2) & 3, pp / 4);
-        });
-      }
-      if constexpr (!(KM_WO_KNOCK & 4)) {
-        static_for<NL>([&](auto l_tag) __attribute__((always_inline)) {
-          constexpr int l = decltype(l_tag)::value;
-          if constexpr (q == at(l, NL, 3 * S / 4 + 1, S)) {
-            if constexpr (l < NS) load_scale_piece(par, s_off, l);
-            else load_code_piece(par, q_off, l - NS);
-          }
-        });
-        if constexpr (q == 3 * S / 4 + 1) load_scalar_scales(par, s + 4);
-      }
+      static_for<16>([&](auto p_tag) __attribute__((always_inline)) {
+        constexpr int pp = decltype(p_tag)::value;
+        if constexpr (NAT && q == at(pp, 16, S / 4, S / 2)) transpose_piece(par, pp);
+      });
+      static_for<4 * UNITS>([&](auto p_tag) __attribute__((always_inline)) {
+        constexpr int pp = decltype(p_tag)::value;
+        if constexpr (q == at(pp, 4 * UNITS, S / 2, 3 * S / 4)) widen_piece(par, pp / 4, pp % 4);
+        if constexpr (pp % 4 == 3 && q == (at(pp, 4 * UNITS, S / 2, 3 * S / 4) + 1 < S ? at(pp, 4 * UNITS, S / 2, 3 * S / 4) + 1 : S - 1)) store_unit((u + 2) & 3, pp / 4);
+      });
+      static_for<NL>([&](auto l_tag) __attribute__((always_inline)) {
+        constexpr int l = decltype(l_tag)::value;
+        if constexpr (q == at(l, NL, L0, S)) {
+          if constexpr (l < NS) load_scale_piece(par, s_off, l);
+          else load_code_piece(par, q_off, l - NS);
+        }
+      });
+      if constexpr (q == L0) load_scalar_scales(par, s + 4);
       // the offsets of the next step's loads, a few instructions each
       if constexpr (q == at(0, 3, S / 2, S)) next_a_off = a_offset(s + 4);
       if constexpr (q == at(1, 3, S / 2, S)) next_q_off = q_offset(s + 5);
       if constexpr (q == at(2, 3, S / 2, S) && NS > 0) next_s_off = scale_offset(s + 5);
       __builtin_amdgcn_sched_barrier(0);
     });
-    WO_STAMP(0);
-    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0((KM_WO_KNOCK & 12) ? 0 : NV));
-    WO_STAMP(1);
+    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(NV));
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
-    WO_STAMP(2);
   };
 
   // prologue: slabs 0 and 1 complete, the A loads of slab 2 done, the codes of slabs 2 and 3 in
@@ -542,9 +522,6 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   for (int r = 0; r < NR; ++r) read_fragment(0, 0, r);
   __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
   __builtin_amdgcn_sched_barrier(0);
-#ifdef KM_WO_STAMPS
-  st_last = wo_cycles();
-#endif
 
   for (int s = 0; s < steps; s += 4) {
     step(std::integral_constant<int, 0>{}, s);
@@ -552,29 +529,41 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
     step(std::integral_constant<int, 2>{}, s + 2);
     step(std::integral_constant<int, 3>{}, s + 3);
   }
-  WO_STAMP(4);
-  // the loads of the padded slabs still in flight write LDS: let them land before the epilogue stages rows there
+  // The loads of the padded slabs are still in flight. Those to LDS must land before the epilogue
+  // stages rows there; those to registers must land before the registers are used for anything
+  // else: to the compiler their results were ready where the load statements stand and are dead
+  // by now, so it would hand the registers to the epilogue at once and the late data would land
+  // on top of accumulator values. Naming them after the wait keeps them allocated until then.
   __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
   __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+#pragma unroll
+    for (int i = 0; i < (NAT ? 8 : 2 * UNITS); ++i) asm volatile("" ::"v"(raw[b][i]));
+#pragma unroll
+    for (int i = 0; i < (NS ? NS : 1); ++i) asm volatile("" ::"v"(sraw[b][i]));
+  }
+  __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  // The MFMAs are opaque statements: nothing tells the compiler that their results take time, and it
+  // copies accumulators to vector registers wherever it likes, the loop exit included. Passing every
+  // accumulator through an (empty) statement placed after the wait makes each later read depend on it.
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) asm volatile("" : "+a"(acc[i][j]));
   __builtin_amdgcn_sched_barrier(0);
 
   // the epilogue stages rows through LDS: half a ring per wavefront
   constexpr int kQuarter = (BM < BN ? BM : BN) * 128;
   static_assert(STAGES * A_STAGE / 2 >= kQuarter && STAGES * B_STAGE / 2 >= kQuarter, "staging room");
   uint8_t* bufs[4] = {a_ring, a_ring + STAGES * A_STAGE / 2, b_ring, b_ring + STAGES * B_STAGE / 2};
-  if constexpr (KM_WO_KNOCK & 32) { if (acc[0][0][0] == 123.f) C[0] = 1; }
-  else if constexpr (MODE == kWoFwd)
+  if constexpr (MODE == kWoFwd)
     store_tile<BM, BN, DT, 1>(acc, 1.0f, nullptr, static_cast<const float*>(scale_ptr), bias, C, M, NO, m0, n0, bufs[0], bufs[1], bufs[2], bufs[3]);
   else if constexpr (MODE == kWoDgradT)
     store_tile<BM, BN, DT, 0>(acc, 1.0f, nullptr, nullptr, nullptr, C, M, NO, m0, n0, bufs[0], bufs[1], bufs[2], bufs[3]);
   else
     store_tile_by_fours<BM, BN, DT>(acc, C, M, NO, m0, n0, bufs[0], bufs[1], bufs[2], bufs[3]);
-#ifdef KM_WO_STAMPS
-  WO_STAMP(5);
-  if (blockIdx.x < 8 && lane == 0)
-    for (int i = 0; i < 8; ++i) g_wo_stamps[(blockIdx.x * 4 + wave) * 8 + i] = st_acc[i];
-#endif
 }
 
 template <int BM, int BN, int DT, int QF, int MODE, int SK>
