@@ -192,7 +192,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_blocks_kernel(
   // every fetch has landed and every wavefront is past its last LDS read: the ring is free
   uint8_t* ea = &a_ring[0][0];
   uint8_t* eb = &b_ring[0][0];
-  store_tile<BM, BN, OUT, 0, false>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, m0, n0, ea, ea + 16384, eb, eb + 16384);
+  store_tile<BM, BN, OUT, 0, false, false>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, m0, n0, ea, ea + 16384, eb, eb + 16384);
 }
 
 struct BlocksConfig {

@@ -13,6 +13,7 @@
 
 namespace km {
 
+
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -140,6 +141,56 @@ __device__ __forceinline__ int fresh_thread_index() {
   return tid;
 }
 
+// The interior-tile path of the epilogues: a wavefront writes its WTM x WTN sub-tile of 16-bit
+// values, 16 rows (one row of MFMA tiles) per pass, through an LDS region of its own of 16 rows
+// of WTN * 2 + 16 bytes. `item(j, t)` yields the 8 bytes of this lane for piece t (0 .. NT-1) of
+// pass j and `col_byte(t)` where they go in the lane's row r16 of the region; the region is read
+// back along rows, 16 bytes a lane, and stored as whole WTN*2-byte row segments (full 128-byte
+// lines) with 16-byte streaming stores (the output is not read again by the kernel and should
+// not push the operand slabs out of L2; plain stores issue twice as fast and make the K loop
+// 15 % slower).
+//
+// One wavefront per SIMD has nothing else to run while it waits, so the passes are pipelined by
+// hand: the transposed rows of pass j are on their way from LDS to registers, and then to memory
+// one store at a time, between the pieces of pass j + 1 as these are read out of the
+// accumulators, rounded and written to LDS. LDS operations of a wavefront execute in order, so
+// pass j + 1 may overwrite the region right behind the reads of pass j. The scheduling barriers
+// keep this order: left alone, the compiler copies all accumulators out first and then has one
+// set of registers for every row, with a full LDS round trip per store.
+template <int WTN, int TM, int NT, class Item, class ColByte>
+__device__ __forceinline__ void staged_rows_out(uint8_t* region, uint8_t* out_base, int N, int lane, Item&& item, ColByte&& col_byte) {
+  constexpr int RP = WTN * 2 + 16;   // LDS row pitch in bytes: the 64 lanes of a write spread evenly over the banks
+  constexpr int LPR = WTN * 2 / 16;  // lanes per row on the read side
+  constexpr int RPI = 64 / LPR;      // rows per read (and store) instruction
+  constexpr int NRD = 16 / RPI;      // reads (and stores) per pass
+  constexpr int kEvery = NT / NRD;   // pieces between two stores
+  static_assert(NT % NRD == 0 && kEvery >= 1, "whole pieces between two stores");
+  const int r16 = lane & 15;
+  const int rd_row = lane / LPR, rd_col = (lane % LPR) * 16;
+  // a uniform row pointer plus a 32-bit lane offset (rd_row < RPI): no 64-bit vector arithmetic per store
+  const uint32_t lane_off = (uint32_t)rd_row * (uint32_t)N * 2u + (uint32_t)rd_col;
+  v4i rd[NRD];
+  auto store_one = [&](int pass, int i) __attribute__((always_inline)) {
+    uint8_t* rows = out_base + (size_t)(pass * 16 + i * RPI) * N * 2;
+    __builtin_nontemporal_store(rd[i], reinterpret_cast<v4i*>(rows + lane_off));
+  };
+  static_for<TM>([&](auto j_tag) __attribute__((always_inline)) {
+    constexpr int j = decltype(j_tag)::value;
+    static_for<NT>([&](auto t_tag) __attribute__((always_inline)) {
+      constexpr int t = decltype(t_tag)::value;
+      *reinterpret_cast<uint2*>(region + r16 * RP + col_byte(t)) = item(j_tag, t_tag);
+      if constexpr (j > 0 && t % kEvery == kEvery - 1) store_one(j - 1, t / kEvery);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+#pragma unroll
+    for (int i = 0; i < NRD; ++i) rd[i] = *reinterpret_cast<const v4i*>(region + (i * RPI + rd_row) * RP + rd_col);
+    __builtin_amdgcn_sched_barrier(0);
+  });
+#pragma unroll
+  for (int i = 0; i < NRD; ++i) store_one(TM - 1, i);
+}
+constexpr int staged_rows_bytes(int wtn) { return 16 * (wtn * 2 + 16); }
+
 // Epilogue of a 2 x 2 wavefront grid over a BM x BN tile of 16x16 MFMA tiles whose rows are
 // output columns: lane (r16 = lane%16, g = lane/16) of tile (t, j) holds
 // C[m0+wm+j*16+r16][n0+wn+t*16+4g .. +3]. Computes acc * post * row_scale[m] * col_scale[n] +
@@ -151,7 +202,21 @@ __device__ __forceinline__ int fresh_thread_index() {
 // A workgroup of eight wavefronts calls it once per group of four (wavefront index modulo 4,
 // m0 of that group's rows) with SYNC off, after a barrier of its own: the groups may take
 // different branches here.
-template <int BM, int BN, int OUT, int SCALED, bool SYNC = true>
+// ACC_AGPR: the accumulators live in AGPRs (kernels whose MFMAs are opaque statements with tied
+// "a" operands). Each element is then copied to a vector register by a statement of its own right
+// where it is consumed, inside its pass; left to the compiler, the 256 copies sit behind the K
+// loop, where they leave no register for anything else.
+template <bool ACC_AGPR>
+__device__ __forceinline__ float acc_element(const v4f& a, int v) {
+  if constexpr (ACC_AGPR) {
+    float r;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(r) : "a"(a[v]));
+    return r;
+  } else {
+    return a[v];
+  }
+}
+template <int BM, int BN, int OUT, int SCALED, bool SYNC = true, bool ACC_AGPR = true>
 __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float post, const float* __restrict__ row_scale,
                                            const float* __restrict__ col_scale, const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N,
                                            int m0, int n0, uint8_t* buf0, uint8_t* buf1, uint8_t* buf2, uint8_t* buf3) {
@@ -176,64 +241,57 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
   };
   if (m0 + BM <= M && n0 + BN <= N && (N & 7) == 0) {
     // Interior tile. A lane holds 4 consecutive n of 16 different rows per MFMA tile; storing
-    // that directly makes 32-byte write requests. Instead each wavefront transposes its
-    // sub-tile through LDS (idle now), 64 rows at a time: 8-byte LDS writes in the MFMA
-    // layout, 16-byte LDS reads along rows, 16-byte global stores that cover whole
-    // WTN*2-byte row segments (full 128-byte lines).
-    constexpr int RP = WTN * 2 + 16;            // LDS row pitch in bytes: 16 lanes x 2 column groups of a write land in 64 different banks
-    constexpr int kMinBuf = (BM < BN ? BM : BN) * 128;
-    constexpr int HM0 = TM < 4 ? TM : 4;        // MFMA tiles (of 16 rows) per pass, halved until
-    constexpr int HM = HM0 * 16 * RP <= kMinBuf ? HM0 : (HM0 / 2) * 16 * RP <= kMinBuf ? HM0 / 2 : 1;  // it fits a buffer
-    constexpr int LPR = WTN * 2 / 16;           // lanes per row on the read side
-    constexpr int RPI = 64 / LPR;               // rows per read instruction
-    static_assert(HM * 16 * RP <= kMinBuf, "epilogue staging: one buffer per wavefront");
+    // that directly makes 32-byte write requests. Each wavefront transposes its sub-tile through
+    // LDS (idle now) instead.
+    static_assert(staged_rows_bytes(WTN) <= (BM < BN ? BM : BN) * 128, "epilogue staging: one buffer per wavefront");
     if constexpr (SYNC) __syncthreads();  // every wavefront is done reading fragments
     uint8_t* region = wave == 0 ? buf0 : wave == 1 ? buf1 : wave == 2 ? buf2 : buf3;
-    const uint16_t* bias_lane = bias + (has_bias ? n0 + wn + 4 * g : 0);
-    float bv[TN][4], cs[TN][4];
-    static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
-      constexpr int t = decltype(t_tag)::value;
-      bv[t][0] = bv[t][1] = bv[t][2] = bv[t][3] = 0.f;
-      cs[t][0] = cs[t][1] = cs[t][2] = cs[t][3] = 1.f;
-      if (col_scale != nullptr) {
-        const float4 c4 = *reinterpret_cast<const float4*>(col_scale + n0 + wn + 4 * g + t * 16);
-        cs[t][0] = c4.x; cs[t][1] = c4.y; cs[t][2] = c4.z; cs[t][3] = c4.w;
-      }
-      if (has_bias) {
-        const uint2 braw = *reinterpret_cast<const uint2*>(bias_lane + t * 16);
-        bv[t][0] = unpack1<OUT>(braw.x & 0xFFFFu); bv[t][1] = unpack1<OUT>(braw.x >> 16);
-        bv[t][2] = unpack1<OUT>(braw.y & 0xFFFFu); bv[t][3] = unpack1<OUT>(braw.y >> 16);
-      }
-    });
-    float rs[TM];
+    uint8_t* out_base = reinterpret_cast<uint8_t*>(C) + ((size_t)(m0 + wm) * N + n0 + wn) * 2;  // uniform
+    auto all_passes = [&](auto bias_tag) __attribute__((always_inline)) {
+      constexpr bool ADD = decltype(bias_tag)::value;
+      float bv[TN][4], cs[TN][4], rs[TM];
+      if constexpr (ADD) {
+        uint2 braw[TN];
 #pragma unroll
-    for (int j = 0; j < TM; ++j) rs[j] = row_scale != nullptr ? post * row_scale[m0 + wm + j * 16 + r16] : post;
-    uint8_t* out_base = reinterpret_cast<uint8_t*>(C) + ((size_t)(m0 + wm) * N + n0 + wn) * 2;
-    const int rd_row = lane / LPR, rd_col = (lane % LPR) * 16;
-    static_for<TM / HM>([&](auto p_tag) __attribute__((always_inline)) {
-      constexpr int pass = decltype(p_tag)::value;
-      static_for<HM>([&](auto j_tag) __attribute__((always_inline)) {
-        constexpr int jj = decltype(j_tag)::value;
-        constexpr int j = pass * HM + jj;
-        static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
-          constexpr int t = decltype(t_tag)::value;
-          float o[4];
+        for (int t = 0; t < TN; ++t) braw[t] = make_uint2(0u, 0u);
+        if (has_bias) {
+          const uint16_t* bias_lane = bias + n0 + wn + 4 * g;
 #pragma unroll
-          for (int v = 0; v < 4; ++v) o[v] = value(acc[t][j][v], rs[j], cs[t][v], bv[t][v]);
-          *reinterpret_cast<uint2*>(region + (jj * 16 + r16) * RP + (t * 16 + 4 * g) * 2) =
-              make_uint2(pack2<OUT>(o[0], o[1]), pack2<OUT>(o[2], o[3]));
-        });
-      });
-      // only this wavefront touches its region: LDS operations of one wavefront stay in order
-      static_for<HM * 16 / RPI>([&](auto i_tag) __attribute__((always_inline)) {
-        constexpr int i = decltype(i_tag)::value;
-        const int row = i * RPI + rd_row;  // within the pass
-        const uint4 v = *reinterpret_cast<const uint4*>(region + row * RP + rd_col);
-        // streaming store: the output is not read again by this kernel and should not push the
-        // operand slabs out of L2
-        __builtin_nontemporal_store(__builtin_bit_cast(v4i, v), reinterpret_cast<v4i*>(out_base + (size_t)(pass * HM * 16 + row) * N * 2 + rd_col));
-      });
-    });
+          for (int t = 0; t < TN; ++t) braw[t] = *reinterpret_cast<const uint2*>(bias_lane + t * 16);
+        }
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+          bv[t][0] = unpack1<OUT>(braw[t].x & 0xFFFFu); bv[t][1] = unpack1<OUT>(braw[t].x >> 16);
+          bv[t][2] = unpack1<OUT>(braw[t].y & 0xFFFFu); bv[t][3] = unpack1<OUT>(braw[t].y >> 16);
+          cs[t][0] = cs[t][1] = cs[t][2] = cs[t][3] = 1.f;
+          if constexpr (SCALED != 0) {
+            if (col_scale != nullptr) {
+              const float4 c4 = *reinterpret_cast<const float4*>(col_scale + n0 + wn + 4 * g + t * 16);
+              cs[t][0] = c4.x; cs[t][1] = c4.y; cs[t][2] = c4.z; cs[t][3] = c4.w;
+            }
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < TM; ++j) rs[j] = (SCALED != 0 && row_scale != nullptr) ? post * row_scale[m0 + wm + j * 16 + r16] : post;
+      }
+      staged_rows_out<WTN, TM, TN>(
+          region, out_base, N, lane,
+          [&](auto j_tag, auto t_tag) __attribute__((always_inline)) {
+            constexpr int j = decltype(j_tag)::value, t = decltype(t_tag)::value;
+            float o[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+              const float a = acc_element<ACC_AGPR>(acc[t][j], v);
+              if constexpr (SCALED == 0 && !ADD) o[v] = a;
+              else o[v] = value(a, rs[j], cs[t][v], bv[t][v]);
+            }
+            return make_uint2(pack2<OUT>(o[0], o[1]), pack2<OUT>(o[2], o[3]));
+          },
+          [&](int t) __attribute__((always_inline)) { return (t * 16 + 4 * g) * 2; });
+    };
+    // without a bias and without scales the accumulator is rounded as it is
+    if (SCALED != 0 || has_bias) all_passes(std::true_type{});
+    else all_passes(std::false_type{});
     return;
   }
   const bool vec_ok = (N & 3) == 0;
@@ -253,7 +311,7 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
       const float rs = row_scale != nullptr ? post * row_scale[m] : post;
       float o[4];
 #pragma unroll
-      for (int v = 0; v < 4; ++v) o[v] = value(acc[t][j][v], rs, cs[v], bv[v]);
+      for (int v = 0; v < 4; ++v) o[v] = value(acc_element<ACC_AGPR>(acc[t][j], v), rs, cs[v], bv[v]);
       uint16_t* dst = C + (size_t)m * N + n;
       if (vec_ok && n + 3 < N) {
         *reinterpret_cast<uint2*>(dst) = make_uint2(pack2<OUT>(o[0], o[1]), pack2<OUT>(o[2], o[3]));

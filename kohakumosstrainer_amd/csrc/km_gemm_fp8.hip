@@ -172,10 +172,6 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
   }
 
   v4f acc[TN][TM];
-#pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
   v8i xf[TM];
   v8i wcur;
@@ -378,17 +374,42 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
   // prologue: A(0), B(0), A(1) (B3: and B(1)) and the scales of step 0
   const uint32_t la0 = lds_offset(a_buf0), la1 = A1 ? la0 : lds_offset(a_buf1);
   const uint32_t lb0 = lds_offset(b_buf0), lb1 = lds_offset(b_buf1), lb2 = lds_offset(b_buf2);
-  dma_a(la0, 0);
-  dma_b(lb0, 0);
+  // The loads of a slab pass through the compute unit's one address unit at 64 bytes a cycle, so
+  // a wavefront that queues them back to back mostly waits to issue: the 256 accumulator
+  // registers are cleared between them. Each accumulator goes through an empty statement that
+  // pins its register writes there (left alone, the compiler sinks them to just in front of the
+  // loop, behind the wait for the slabs).
+  {
+    constexpr int kPasses = A_LD + B_LD, kTiles = TN * TM;
+    const int koff0 = __builtin_amdgcn_readfirstlane(0);
+    static_for<kPasses>([&](auto i_tag) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_tag)::value;
+      if constexpr (i < A_LD) dma_a_pass(la0, koff0, i);
+      else dma_b_pass(lb0, koff0, i - A_LD);
+      static_for<kTiles>([&](auto q_tag) __attribute__((always_inline)) {
+        constexpr int q = decltype(q_tag)::value;
+        if constexpr (q * kPasses / kTiles == i) {
+          acc[q / TM][q % TM] = v4f{0.f, 0.f, 0.f, 0.f};
+          asm volatile("" : "+a"(acc[q / TM][q % TM]));
+        }
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  }
   scale_fetch(0);
-  if constexpr (!A1) dma_a(la1, min(1, nk - 1));
   if constexpr (B3) {
+    dma_a(la1, min(1, nk - 1));
     dma_b(lb1, min(1, nk - 1), I8 && nk < 2 ? (int)0x80000000 : 0);
     scale_touch(min(1, nk - 1), lb2);
     scale_touch(min(2, nk - 1), lb2);
   }
   __builtin_amdgcn_s_waitcnt(kWaitVm0);
+  __builtin_amdgcn_sched_barrier(0);
   __syncthreads();
+  // The second A slab is not needed before the end of step 0, whose closing wait leaves in flight
+  // only as many loads as the A passes that step issues itself: requested here, behind the wait
+  // for the first slabs, its passes find the address unit idle.
+  if constexpr (!A1 && !B3) dma_a(la1, min(1, nk - 1));
   if constexpr (!I8) scale_commit(set0_t{}, 0xFFFFFFFFu);
 #pragma unroll
   for (int j = 0; j < TM; ++j) xf[j] = fragment(la0, wm + j * 16 + r16);
@@ -416,19 +437,11 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
   }
   __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));  // the last (clamped) prefetches and fragment reads must be done before LDS is reused
 
-  // the MFMAs above are opaque to the compiler's hazard handling: give the last ones time to
-  // retire before the accumulators are read
+  // The MFMAs above are opaque to the compiler's hazard handling: give the last ones time to
+  // retire before the accumulators are read. The epilogue reads every accumulator element with an
+  // opaque statement of its own, which stays behind this one.
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
-  // The compiler does not know that the opaque MFMAs' results take time and copies accumulators to
-  // vector registers wherever it likes (the loop exit included): passing every accumulator through an
-  // empty statement placed after the wait makes each later read depend on it.
-#pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j) asm volatile("" : "+a"(acc[i][j]));
-  __builtin_amdgcn_sched_barrier(0);
-
   // epilogue: bias (and the per-tensor scales) on the fp32 accumulator, one rounding
   float post = 1.0f;
   const float *row_scale = nullptr, *col_scale = nullptr;

@@ -100,40 +100,24 @@ __device__ __forceinline__ void store_tile_by_fours(v4f (&acc)[BN / 32][BM / 32]
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6) & 3;
   const int wm = (wave >> 1) * WTM, wn = (wave & 1) * WTN;
   const int r16 = lane & 15, g = lane >> 4;
+  // every accumulator element is read by an opaque statement at its use (see store_tile)
   auto four = [&](int b, int j, int v) __attribute__((always_inline)) {
-    return make_uint2(pack2<OUT>(acc[b][j][v], acc[Q + b][j][v]), pack2<OUT>(acc[2 * Q + b][j][v], acc[3 * Q + b][j][v]));
+    return make_uint2(pack2<OUT>(acc_element<true>(acc[b][j], v), acc_element<true>(acc[Q + b][j], v)),
+                      pack2<OUT>(acc_element<true>(acc[2 * Q + b][j], v), acc_element<true>(acc[3 * Q + b][j], v)));
   };
   if (m0 + BM <= M && n0 + BN <= NO && (NO & 7) == 0) {
-    constexpr int RP = WTN * 2 + 16;
-    constexpr int kMinBuf = (BM < BN ? BM : BN) * 128;
-    constexpr int HM0 = TM < 4 ? TM : 4;
-    constexpr int HM = HM0 * 16 * RP <= kMinBuf ? HM0 : (HM0 / 2) * 16 * RP <= kMinBuf ? HM0 / 2 : 1;
-    constexpr int LPR = WTN * 2 / 16;  // lanes per row on the read side
-    constexpr int RPI = 64 / LPR;      // rows per read instruction
-    static_assert(HM * 16 * RP <= kMinBuf, "epilogue staging: one buffer per wavefront");
+    static_assert(staged_rows_bytes(WTN) <= (BM < BN ? BM : BN) * 128, "epilogue staging: one buffer per wavefront");
     __syncthreads();  // every wavefront is done reading fragments
     uint8_t* region = wave == 0 ? buf0 : wave == 1 ? buf1 : wave == 2 ? buf2 : buf3;
     uint8_t* out_base = reinterpret_cast<uint8_t*>(C) + ((size_t)(m0 + wm) * NO + n0 + wn) * 2;
-    const int rd_row = lane / LPR, rd_col = (lane % LPR) * 16;
-    static_for<TM / HM>([&](auto p_tag) __attribute__((always_inline)) {
-      constexpr int pass = decltype(p_tag)::value;
-      static_for<HM>([&](auto j_tag) __attribute__((always_inline)) {
-        constexpr int jj = decltype(j_tag)::value;
-        constexpr int j = pass * HM + jj;
-#pragma unroll
-        for (int b = 0; b < Q; ++b)
-#pragma unroll
-          for (int v = 0; v < 4; ++v)
-            *reinterpret_cast<uint2*>(region + (jj * 16 + r16) * RP + (64 * b + 16 * g + 4 * v) * 2) = four(b, j, v);
-      });
-      // only this wavefront touches its region: LDS operations of one wavefront stay in order
-      static_for<HM * 16 / RPI>([&](auto i_tag) __attribute__((always_inline)) {
-        constexpr int i = decltype(i_tag)::value;
-        const int row = i * RPI + rd_row;  // within the pass
-        const uint4 val = *reinterpret_cast<const uint4*>(region + row * RP + rd_col);
-        __builtin_nontemporal_store(__builtin_bit_cast(v4i, val), reinterpret_cast<v4i*>(out_base + (size_t)(pass * HM * 16 + row) * NO * 2 + rd_col));
-      });
-    });
+    // piece t = 4 b + v of a pass: the columns 64 b + 16 g + 4 v .. + 3 of this lane's row
+    staged_rows_out<WTN, TM, 4 * Q>(
+        region, out_base, NO, lane,
+        [&](auto j_tag, auto t_tag) __attribute__((always_inline)) {
+          constexpr int j = decltype(j_tag)::value, t = decltype(t_tag)::value;
+          return four(t / 4, j, t % 4);
+        },
+        [&](int t) __attribute__((always_inline)) { return (64 * (t / 4) + 16 * g + 4 * (t % 4)) * 2; });
     return;
   }
 #pragma unroll
@@ -287,10 +271,6 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   const int b_frag = lds_offset(b_ring) + slab32_offset(wn + r16, g);  // + t KiB + stage
 
   v4f acc[TN][TM];
-#pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
   // codes and scales in flight, set s & 1 for slab s
   uint32_t raw[2][NAT ? 8 : 2 * UNITS];
@@ -506,6 +486,17 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   dma_a(2, 2);
   load_slab(0, 0);
   load_slab(1, 1);
+  // The accumulators are cleared while the first loads are on their way: each one goes through an
+  // empty statement that pins its register writes here (left alone, the compiler sinks them to
+  // just in front of the loop, behind the waits).
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+      asm volatile("" : "+a"(acc[i][j]));
+    }
+  __builtin_amdgcn_sched_barrier(0);
   // The optimizer takes the result of a load statement for ready where the statement stands: nothing
   // that reads it may move above the wait (in the steps every slot ends in a scheduling barrier).
   __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
@@ -545,13 +536,9 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   }
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
-  // The MFMAs are opaque statements: nothing tells the compiler that their results take time, and it
-  // copies accumulators to vector registers wherever it likes, the loop exit included. Passing every
-  // accumulator through an (empty) statement placed after the wait makes each later read depend on it.
-#pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j) asm volatile("" : "+a"(acc[i][j]));
+  // The MFMAs are opaque statements: nothing tells the compiler that their results take time. The
+  // epilogues read every accumulator element with an opaque statement of its own, which stays
+  // behind the wait above in program order.
   __builtin_amdgcn_sched_barrier(0);
 
   // the epilogue stages rows through LDS: half a ring per wavefront
