@@ -216,7 +216,9 @@ __device__ __forceinline__ float acc_element(const v4f& a, int v) {
     return a[v];
   }
 }
-template <int BM, int BN, int OUT, int SCALED, bool SYNC = true, bool ACC_AGPR = true>
+// CLEAR: every accumulator is set to zero once it has been read (a work-group that goes on to
+// another tile starts its K loop without a pass over the 256 registers).
+template <int BM, int BN, int OUT, int SCALED, bool SYNC = true, bool ACC_AGPR = true, bool CLEAR = false>
 __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float post, const float* __restrict__ row_scale,
                                            const float* __restrict__ col_scale, const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N,
                                            int m0, int n0, uint8_t* buf0, uint8_t* buf1, uint8_t* buf2, uint8_t* buf3) {
@@ -243,7 +245,7 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
     // Interior tile. A lane holds 4 consecutive n of 16 different rows per MFMA tile; storing
     // that directly makes 32-byte write requests. Each wavefront transposes its sub-tile through
     // LDS (idle now) instead.
-    static_assert(staged_rows_bytes(WTN) <= (BM < BN ? BM : BN) * 128, "epilogue staging: one buffer per wavefront");
+    // (each of the four buffers holds staged_rows_bytes(WTN) bytes)
     if constexpr (SYNC) __syncthreads();  // every wavefront is done reading fragments
     uint8_t* region = wave == 0 ? buf0 : wave == 1 ? buf1 : wave == 2 ? buf2 : buf3;
     uint8_t* out_base = reinterpret_cast<uint8_t*>(C) + ((size_t)(m0 + wm) * N + n0 + wn) * 2;  // uniform
@@ -285,6 +287,10 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
               if constexpr (SCALED == 0 && !ADD) o[v] = a;
               else o[v] = value(a, rs[j], cs[t][v], bv[t][v]);
             }
+            if constexpr (CLEAR) {
+              acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+              asm volatile("" : "+a"(acc[t][j]));
+            }
             return make_uint2(pack2<OUT>(o[0], o[1]), pack2<OUT>(o[2], o[3]));
           },
           [&](int t) __attribute__((always_inline)) { return (t * 16 + 4 * g) * 2; });
@@ -321,6 +327,15 @@ __device__ __forceinline__ void store_tile(v4f (&acc)[BN / 32][BM / 32], float p
           if (n + v < N) dst[v] = (uint16_t)(pack2<OUT>(o[v], 0.f) & 0xFFFFu);
       }
     }
+  }
+  if constexpr (CLEAR) {
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+      for (int j = 0; j < TM; ++j) {
+        acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+        asm volatile("" : "+a"(acc[t][j]));
+      }
   }
 }
 
