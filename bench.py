@@ -121,9 +121,9 @@ def other_configs(dev, reps):
             d_ms[cfg] = event_ms(lambda: native.wo_gemm_dgrad(dy, q, scale, cfg), reps)
         (fc, f), (dc, d) = min(f_ms.items(), key=lambda kv: kv[1]), min(d_ms.items(), key=lambda kv: kv[1])
         flop = 2 * m * n * k
-        # a rotated base (ConvRot, groups of 128) adds one rotation pass over x in forward and one over dx in the input gradient
-        native.group_hadamard(x, 128)
-        r = event_ms(lambda: native.group_hadamard(x, 128), reps)
+        # a rotated base (ConvRot, groups of 256) adds one rotation pass over x in forward and one over dx in the input gradient
+        native.group_hadamard(x, 256)
+        r = event_ms(lambda: native.group_hadamard(x, 256), reps)
         out[name] = {"fwd_ms": f, "fwd_TFLOPs": flop / f / 1e9, "fwd_config": fc, "dgrad_ms": d, "dgrad_TFLOPs": flop / d / 1e9, "dgrad_config": dc,
                      "peak_TFLOPs": 2500.0, "note": "dgrad reads the codes as stored: no transposed copy, no workspace",
                      "rotation_pass_ms": r, "rotation_share_of_rotated_fwd": r / (r + f), "rotation_share_of_rotated_dgrad": r / (r + d)}

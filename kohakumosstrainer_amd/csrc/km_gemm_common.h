@@ -144,7 +144,8 @@ __device__ __forceinline__ int fresh_thread_index() {
 // The interior-tile path of the epilogues: a wavefront writes its WTM x WTN sub-tile of 16-bit
 // values, 16 rows (one row of MFMA tiles) per pass, through an LDS region of its own of 16 rows
 // of WTN * 2 + 16 bytes. `item(j, t)` yields the 8 bytes of this lane for piece t (0 .. NT-1) of
-// pass j and `col_byte(t)` where they go in the lane's row r16 of the region; the region is read
+// pass j and `col_byte(t)` where they go in the lane's row r16 of the region (negative: the lane
+// has no such piece); the region is read
 // back along rows, 16 bytes a lane, and stored as whole WTN*2-byte row segments (full 128-byte
 // lines) with 16-byte streaming stores (the output is not read again by the kernel and should
 // not push the operand slabs out of L2; plain stores issue twice as fast and make the K loop
@@ -160,30 +161,38 @@ __device__ __forceinline__ int fresh_thread_index() {
 template <int WTN, int TM, int NT, class Item, class ColByte>
 __device__ __forceinline__ void staged_rows_out(uint8_t* region, uint8_t* out_base, int N, int lane, Item&& item, ColByte&& col_byte) {
   constexpr int RP = WTN * 2 + 16;   // LDS row pitch in bytes: the 64 lanes of a write spread evenly over the banks
-  constexpr int LPR = WTN * 2 / 16;  // lanes per row on the read side
-  constexpr int RPI = 64 / LPR;      // rows per read (and store) instruction
-  constexpr int NRD = 16 / RPI;      // reads (and stores) per pass
-  constexpr int kEvery = NT / NRD;   // pieces between two stores
-  static_assert(NT % NRD == 0 && kEvery >= 1, "whole pieces between two stores");
+  constexpr int LPR = WTN * 2 / 16;  // 16-byte pieces per row on the read side
+  constexpr int NRD = 16 * LPR / 64; // reads (and stores) per pass: the pass's 16 LPR pieces, 64 per instruction
+  static_assert((16 * LPR) % 64 == 0 && NT >= NRD, "whole instructions per pass, at least a piece between two stores");
   const int r16 = lane & 15;
-  const int rd_row = lane / LPR, rd_col = (lane % LPR) * 16;
-  // a uniform row pointer plus a 32-bit lane offset (rd_row < RPI): no 64-bit vector arithmetic per store
-  const uint32_t lane_off = (uint32_t)rd_row * (uint32_t)N * 2u + (uint32_t)rd_col;
+  // piece 64 i + lane of a pass is (row, 16-byte column) = (piece / LPR, piece % LPR): its LDS offset
+  // and its offset from the pass's first output row, 32 bits (row < 16): a uniform row pointer per
+  // pass and no 64-bit vector arithmetic per store
+  uint32_t lds_off[NRD], out_off[NRD];
+#pragma unroll
+  for (int i = 0; i < NRD; ++i) {
+    const int piece = i * 64 + lane;
+    lds_off[i] = (uint32_t)((piece / LPR) * RP + (piece % LPR) * 16);
+    out_off[i] = (uint32_t)(piece / LPR) * (uint32_t)N * 2u + (uint32_t)(piece % LPR) * 16u;
+  }
   v4i rd[NRD];
   auto store_one = [&](int pass, int i) __attribute__((always_inline)) {
-    uint8_t* rows = out_base + (size_t)(pass * 16 + i * RPI) * N * 2;
-    __builtin_nontemporal_store(rd[i], reinterpret_cast<v4i*>(rows + lane_off));
+    uint8_t* rows = out_base + (size_t)(pass * 16) * N * 2;
+    __builtin_nontemporal_store(rd[i], reinterpret_cast<v4i*>(rows + out_off[i]));
   };
   static_for<TM>([&](auto j_tag) __attribute__((always_inline)) {
     constexpr int j = decltype(j_tag)::value;
     static_for<NT>([&](auto t_tag) __attribute__((always_inline)) {
       constexpr int t = decltype(t_tag)::value;
-      *reinterpret_cast<uint2*>(region + r16 * RP + col_byte(t)) = item(j_tag, t_tag);
-      if constexpr (j > 0 && t % kEvery == kEvery - 1) store_one(j - 1, t / kEvery);
+      const uint2 piece = item(j_tag, t_tag);
+      const int at = col_byte(t);  // negative: this lane has no piece t
+      if (at >= 0) *reinterpret_cast<uint2*>(region + r16 * RP + at) = piece;
+      // store i of the pass before goes behind piece (i + 1) NT / NRD - 1
+      if constexpr (j > 0 && ((t + 1) * NRD) / NT > (t * NRD) / NT) store_one(j - 1, (t * NRD) / NT);
       __builtin_amdgcn_sched_barrier(0);
     });
 #pragma unroll
-    for (int i = 0; i < NRD; ++i) rd[i] = *reinterpret_cast<const v4i*>(region + (i * RPI + rd_row) * RP + rd_col);
+    for (int i = 0; i < NRD; ++i) rd[i] = *reinterpret_cast<const v4i*>(region + lds_off[i]);
     __builtin_amdgcn_sched_barrier(0);
   });
 #pragma unroll

@@ -87,7 +87,7 @@ __global__ __launch_bounds__(256) void transpose_bytes(const uint8_t* __restrict
 struct WoConfig {
   int bm, bn;
 };
-static const WoConfig kWoConfigs[] = {{256, 256}, {128, 256}, {256, 128}, {128, 128}, {64, 128}};
+static const WoConfig kWoConfigs[] = {{256, 256}, {128, 256}, {256, 128}, {128, 128}, {64, 128}, {256, 192}};
 static_assert(sizeof(kWoConfigs) / sizeof(kWoConfigs[0]) == kNumWoConfigs, "one row per case of launch_config");
 
 int wo_num_configs() { return kNumWoConfigs; }

@@ -87,14 +87,20 @@ __device__ __forceinline__ void transpose_8x4(const uint32_t (&d)[8], uint2 (&o)
 // Epilogue of the input-gradient kernel that reads q as stored. Row 16 t + r of a wavefront's B
 // slab holds column 64 b + 4 r + j of the wavefront's WTN columns, t = j Q + b, Q = WTN / 64: lane
 // (r16, g) holds, for every b, the sixteen consecutive columns 64 b + 16 g .. + 15 of output row
-// r16, element v of tile j Q + b being column 64 b + 16 g + 4 v + j. Interior tiles go through
-// the same LDS staging as store_tile (8-byte LDS writes, 16-byte reads along rows, full-line
-// global stores); edge tiles store four columns at a time (NO % 4 == 0 here). No scale, no bias.
+// r16, element v of tile j Q + b being column 64 b + 16 g + 4 v + j. A 96-column wavefront has
+// tiles 0-3 laid out like that (b = 0) and its columns 64 .. 95 in tiles 4 and 5: row i of tile 4
+// is column 64 + 4 (i % 8) + i / 8, of tile 5 column 64 + 4 (i % 8) + 2 + i / 8, so the lower 32
+// lanes hold residues 0 and 2 of columns 64 + 16 g + 4 v .. + 3 and the lanes 32 places up
+// residues 1 and 3: V_PERMLANE32_SWAP brings them together and the lower lanes write the piece.
+// Interior tiles go through the same LDS staging as store_tile (8-byte LDS writes, 16-byte reads
+// along rows, full-line global stores); edge tiles store four columns at a time (NO % 4 == 0
+// here). No scale, no bias.
 template <int BM, int BN, int OUT>
 __device__ __forceinline__ void store_tile_by_fours(v4f (&acc)[BN / 32][BM / 32], uint16_t* __restrict__ C, int M, int NO, int m0,
                                                     int n0, uint8_t* buf0, uint8_t* buf1, uint8_t* buf2, uint8_t* buf3) {
   constexpr int WTM = BM / 2, WTN = BN / 2, TM = WTM / 16, Q = WTN / 64;
-  static_assert(BN / 32 == 4 * Q, "four column residues per 64 columns");
+  constexpr bool kTail = WTN % 64 != 0;  // 32 more columns in the last two tiles
+  static_assert(BN / 32 == 4 * Q + (kTail ? 2 : 0) && (!kTail || WTN % 64 == 32), "four column residues per 64 columns");
   const int tid = fresh_thread_index();  // see store_tile
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6) & 3;
@@ -105,19 +111,29 @@ __device__ __forceinline__ void store_tile_by_fours(v4f (&acc)[BN / 32][BM / 32]
     return make_uint2(pack2<OUT>(acc_element<true>(acc[b][j], v), acc_element<true>(acc[Q + b][j], v)),
                       pack2<OUT>(acc_element<true>(acc[2 * Q + b][j], v), acc_element<true>(acc[3 * Q + b][j], v)));
   };
+  // the piece of the tail tiles: valid in the lower 32 lanes (g < 2), columns 64 Q + 16 g + 4 v .. + 3
+  auto tail_four = [&](int j, int v) __attribute__((always_inline)) {
+    const uint32_t x = __builtin_bit_cast(uint32_t, acc_element<true>(acc[4 * Q][j], v));
+    const uint32_t y = __builtin_bit_cast(uint32_t, acc_element<true>(acc[4 * Q + 1][j], v));
+    const auto xs = __builtin_amdgcn_permlane32_swap(x, x, false, false);  // [1]: the value 32 lanes up
+    const auto ys = __builtin_amdgcn_permlane32_swap(y, y, false, false);
+    return make_uint2(pack2<OUT>(__builtin_bit_cast(float, x), __builtin_bit_cast(float, (uint32_t)xs[1])),
+                      pack2<OUT>(__builtin_bit_cast(float, y), __builtin_bit_cast(float, (uint32_t)ys[1])));
+  };
   if (m0 + BM <= M && n0 + BN <= NO && (NO & 7) == 0) {
-    static_assert(staged_rows_bytes(WTN) <= (BM < BN ? BM : BN) * 128, "epilogue staging: one buffer per wavefront");
     __syncthreads();  // every wavefront is done reading fragments
     uint8_t* region = wave == 0 ? buf0 : wave == 1 ? buf1 : wave == 2 ? buf2 : buf3;
     uint8_t* out_base = reinterpret_cast<uint8_t*>(C) + ((size_t)(m0 + wm) * NO + n0 + wn) * 2;
-    // piece t = 4 b + v of a pass: the columns 64 b + 16 g + 4 v .. + 3 of this lane's row
-    staged_rows_out<WTN, TM, 4 * Q>(
+    // piece t = 4 b + v of a pass: the columns 64 b + 16 g + 4 v .. + 3 of this lane's row; the
+    // four pieces after those are the tail's (no write from the upper lanes: offset -1)
+    staged_rows_out<WTN, TM, 4 * Q + (kTail ? 4 : 0)>(
         region, out_base, NO, lane,
         [&](auto j_tag, auto t_tag) __attribute__((always_inline)) {
           constexpr int j = decltype(j_tag)::value, t = decltype(t_tag)::value;
-          return four(t / 4, j, t % 4);
+          if constexpr (t < 4 * Q) return four(t / 4, j, t % 4);
+          else return tail_four(j, t - 4 * Q);
         },
-        [&](int t) __attribute__((always_inline)) { return (64 * (t / 4) + 16 * g + 4 * (t % 4)) * 2; });
+        [&](int t) __attribute__((always_inline)) { return t < 4 * Q ? (64 * (t / 4) + 16 * g + 4 * (t % 4)) * 2 : g < 2 ? (64 * Q + 16 * g + 4 * (t - 4 * Q)) * 2 : -1; });
     return;
   }
 #pragma unroll
@@ -128,8 +144,17 @@ __device__ __forceinline__ void store_tile_by_fours(v4f (&acc)[BN / 32][BM / 32]
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int col = n0 + wn + 64 * b + 16 * g + 4 * v;
-        if (m < M && col < NO) *reinterpret_cast<uint2*>(C + (size_t)m * NO + col) = four(b, j, v);
+        const uint2 piece = four(b, j, v);
+        if (m < M && col < NO) *reinterpret_cast<uint2*>(C + (size_t)m * NO + col) = piece;
       }
+    if constexpr (kTail) {
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int col = n0 + wn + 64 * Q + 16 * g + 4 * v;
+        const uint2 piece = tail_four(j, v);  // every lane takes part in the exchange
+        if (g < 2 && m < M && col < NO) *reinterpret_cast<uint2*>(C + (size_t)m * NO + col) = piece;
+      }
+    }
   }
 }
 
@@ -230,7 +255,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   constexpr int NQ = NAT ? 8 : UNITS;                  // code loads per thread and step
   constexpr int NS = !NAT ? 0 : SK == KM_WSCALE_E8M0 ? 8 : SK == KM_WSCALE_BLOCKS ? 1 : 0;  // scale loads through the vector path
   constexpr int NV = A_LD + NQ + NS;                   // vector-memory loads issued per step, counted by hand below
-  static_assert(!NAT || BN == 256 || BN == 128, "the transposing load covers 256 or 128 columns");
+  static_assert(!NAT || BN == 256 || BN == 192 || BN == 128, "the transposing load covers 256, 192 or 128 columns");
   static_assert(NV < 48, "vmcnt holds 6 bits");
   __shared__ __attribute__((aligned(1024))) uint8_t a_ring[STAGES * A_STAGE];
   __shared__ __attribute__((aligned(1024))) uint8_t b_ring[STAGES * B_STAGE];
@@ -265,7 +290,13 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   const bool nat_live = lane < LPR;
   const int col4 = lane % LPR;                               // columns 4 col4 .. 4 col4 + 3 of the tile
   const int half_w = col4 / (LPR / 2), col_l = col4 % (LPR / 2);
-  const int nat_row0 = half_w * WTN + col_l;                 // slab row of column j: nat_row0 + j * (WTN / 4)
+  // slab row of column j: nat_row0 + j * nat_stride. A wavefront's WTN / 4 dwords per row n are laid
+  // out so that every 16-row MFMA tile holds one j: with WTN / 4 a multiple of 16, j-major; with the
+  // 24 dwords of a 96-column half, dwords 0-15 j-major in tiles 0-3 and dwords 16-23 as rows
+  // 64 + 8 j + (dword - 16) of tiles 4 and 5 (see store_tile_by_fours)
+  constexpr bool kNatWhole = (WTN / 4) % 16 == 0;
+  const int nat_row0 = half_w * WTN + (kNatWhole || col_l < 16 ? col_l : 48 + col_l);
+  const int nat_stride = kNatWhole ? WTN / 4 : col_l < 16 ? 16 : 8;
 
   const int a_frag = lds_offset(a_ring) + slab32_offset(wm + r16, g);  // + j KiB + stage
   const int b_frag = lds_offset(b_ring) + slab32_offset(wn + r16, g);  // + t KiB + stage
@@ -392,7 +423,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
     uint8_t* slab = b_ring + stage * B_STAGE;
     const uint4 v = make_uint4(w16[c][0], w16[c][1], w16[c][2], w16[c][3]);
     if constexpr (!NAT) *reinterpret_cast<uint4*>(slab + slab32_offset(q_row + c * 64, q_chunk)) = v;
-    else if (nat_live) *reinterpret_cast<uint4*>(slab + slab32_offset(nat_row0 + c * (WTN / 4), wave)) = v;
+    else if (nat_live) *reinterpret_cast<uint4*>(slab + slab32_offset(nat_row0 + c * nat_stride, wave)) = v;
   };
   auto commit_all = [&](int set, int stage) __attribute__((always_inline)) {
 #pragma unroll
@@ -542,8 +573,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   __builtin_amdgcn_sched_barrier(0);
 
   // the epilogue stages rows through LDS: half a ring per wavefront
-  constexpr int kQuarter = (BM < BN ? BM : BN) * 128;
-  static_assert(STAGES * A_STAGE / 2 >= kQuarter && STAGES * B_STAGE / 2 >= kQuarter, "staging room");
+  static_assert(STAGES * A_STAGE / 2 >= staged_rows_bytes(WTN) && STAGES * B_STAGE / 2 >= staged_rows_bytes(WTN), "staging room");
   uint8_t* bufs[4] = {a_ring, a_ring + STAGES * A_STAGE / 2, b_ring, b_ring + STAGES * B_STAGE / 2};
   if constexpr (MODE == kWoFwd)
     store_tile<BM, BN, DT, 1>(acc, 1.0f, nullptr, static_cast<const float*>(scale_ptr), bias, C, M, NO, m0, n0, bufs[0], bufs[1], bufs[2], bufs[3]);
@@ -571,6 +601,11 @@ inline int launch_config(int config, const void* a, const void* q, const void* s
     case 2: return launch_wo<256, 128, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st);
     case 3: return launch_wo<128, 128, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st);
     case 4: return launch_wo<64, 128, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st);
+    case 5:
+      // 192 columns: whole waves of tiles where 256-column tiles leave compute units idle (3072
+      // output columns: 16 x 16 = 256 tiles against 16 x 12 = 192 at M = 4096, 32 x 16 = 512 against
+      // 32 x 12 = 384 at M = 8192)
+      return launch_wo<256, 192, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st);
   }
   return km_fail(KM_ERR_ARG, "km_wo_gemm: unknown config");
 }

@@ -97,3 +97,35 @@ def test_int8_gemm_walks_tiles(m, n, k):
     acc = (a[rows].double() @ b.double().T).float()  # exact: |sum| < 2^24 * 2^7
     want = (((acc * sa[rows, None]) * sb[None, :]) + bias.float()).to(torch.bfloat16)
     assert torch.equal(y[rows.cuda()].cpu(), want)
+
+
+def test_resident_launch_under_graph_capture():
+    """The first launch of a configuration asks the runtime how many work-groups the card holds;
+    that query and the launch itself must work while a stream is being captured, and every replay
+    must give the eager result (inputs refilled between replays, eager work in between)."""
+    m, n, k = 4096, 4352, 256  # 16 x 17 = 272 tiles of 256 x 256: more than the card's compute units
+    g = torch.Generator().manual_seed(21)
+    dev = torch.device("cuda:0")
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(n, k, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    wq, _, wsp = native.quant_mx(w, natural=False, packed=True)
+    static_x = x.clone()
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        for cfg in (2, 0):  # warm both paths outside the capture as a training loop would
+            xq, _, xsp = native.quant_mx(static_x, natural=False, packed=True)
+            native.gemm_mx(xq, xsp, wq, wsp, None, torch.bfloat16, cfg, packed=True)
+    torch.cuda.current_stream().wait_stream(stream)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        xq, _, xsp = native.quant_mx(static_x, natural=False, packed=True)
+        y_graph = native.gemm_mx(xq, xsp, wq, wsp, None, torch.bfloat16, 0, packed=True)
+    for i in range(3):
+        fresh = torch.randn(m, k, generator=g).to(torch.bfloat16).to(dev) * (i + 1)
+        static_x.copy_(fresh)
+        graph.replay()
+        xq, _, xsp = native.quant_mx(fresh, natural=False, packed=True)
+        eager = native.gemm_mx(xq, xsp, wq, wsp, None, torch.bfloat16, 0, packed=True)
+        torch.cuda.synchronize()
+        assert torch.equal(y_graph, eager), f"replay {i}"

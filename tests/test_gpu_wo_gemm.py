@@ -12,7 +12,7 @@ from oracle import linear
 from oracle.stats import assert_no_regression, rel_l2
 
 pytestmark = pytest.mark.gpu
-SHAPES = ((200, 150, 136), (1, 96, 64), (513, 384, 1000), (300, 256, 512), (1024, 512, 256))
+SHAPES = ((200, 150, 136), (1, 96, 64), (513, 384, 1000), (300, 256, 512), (1024, 512, 256), (512, 320, 768))
 
 
 def must_fail(check, what=""):
