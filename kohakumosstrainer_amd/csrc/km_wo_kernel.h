@@ -208,12 +208,15 @@ enum { kWoFwd = 0, kWoDgradT = 1, kWoDgradN = 2 };
 // kWoDgradN  codes [KC, NO] (q as stored); scale(n, k) by SK, applied before the rounding
 
 // LDS layout of a 32-deep slab: a row is 64 bytes (four 16-byte chunks of eight 16-bit values),
-// sixteen rows fill 1 KiB. Rows r and r+4 of a 16-row block differ in the 256-byte line, rows that
-// differ in r % 4 in the 64-byte quarter of it, and the chunk index is XORed with (r / 4) % 4: the
-// 16 lanes (16 rows, one chunk) of an MFMA fragment read hit 16 different 16-byte slots modulo 256
-// bytes, and so do 16 lanes that write four chunks of four consecutive rows.
+// rows in order, sixteen rows fill 1 KiB; the chunk index is XORed with (row / 2) % 4. A 16-byte
+// LDS access is served eight lanes at a time, 128 bytes a cycle: eight consecutive lanes must hit
+// eight different 16-byte slots modulo 128 bytes. Eight lanes that read one chunk of eight
+// consecutive rows (an MFMA fragment read, or the transposing mode's writes) do: two rows share a
+// 128-byte line and the four lines differ in the XOR key; so do eight lanes that write the four
+// chunks of two consecutive rows. (A layout that spread 16 lanes over 256 bytes instead measured
+// bank conflicts in 40-50 % of the LDS-active cycles.)
 __device__ __forceinline__ int slab32_offset(int row, int chunk) {
-  return ((row >> 4) << 10) + (((row >> 2) & 3) << 8) + ((row & 3) << 6) + ((chunk ^ ((row >> 2) & 3)) << 4);
+  return (row << 6) + ((chunk ^ ((row >> 1) & 3)) << 4);
 }
 
 // In-loop forms without the wait states for a vector-ALU-written SGPR: inside the K loop every SGPR
@@ -278,9 +281,9 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   const v4i q_rsrc = raw_rsrc(Q + q_skip, (uint32_t)min((int64_t)NO * KC - q_skip, (int64_t)0x7FFFFFFF));
 
   // direct-to-LDS A pass: lane L lands in 16-byte slot L of its wavefront's 1 KiB block, which is
-  // (row 4 (L / 16) + (L % 16) / 4, chunk (L % 4) ^ (L / 16)) of the block in the slab layout
-  const int dma_row = wave * 16 + ((lane >> 4) << 2) + ((lane & 15) >> 2);
-  const int dma_chunk = (lane & 3) ^ (lane >> 4);
+  // (row L / 4, chunk (L % 4) ^ (L / 8) % 4) of the block in the slab layout
+  const int dma_row = wave * 16 + (lane >> 2);
+  const int dma_chunk = (lane & 3) ^ ((lane >> 3) & 3);
   // K-contiguous codes: four lanes cover the 32 codes of a row, a wavefront 16 rows, a unit 64 rows
   const int q_row = wave * 16 + (lane >> 2), q_chunk = lane & 3;
   // codes as stored: LPR lanes cover the BN columns of one row n with a dword each (the other lanes
