@@ -183,6 +183,13 @@ def test_int8_weight_only_frozen_base_shape():
     assert rel_l2(y[rows].cpu(), truth) <= 2e-3
     perm = torch.randperm(m, generator=g).cuda()
     assert torch.equal(native.wo_gemm_fwd(xg[perm].contiguous(), qg, sg, bg, 0), y[perm])
+    # every tile shape (the 192-column one fills the card exactly at this shape) adds a row's
+    # products in the same order
+    dy = torch.randn(m, n, generator=g).to(torch.bfloat16).cuda()
+    dx = native.wo_gemm_dgrad(dy, qg, sg, 0)
+    for cfg in range(1, n_configs()):
+        assert torch.equal(native.wo_gemm_fwd(xg, qg, sg, bg, cfg), y), f"forward cfg{cfg}"
+        assert torch.equal(native.wo_gemm_dgrad(dy, qg, sg, cfg), dx), f"input gradient cfg{cfg}"
 
 
 def test_fp8_weight_only_per_tensor_scale_mlp_up_projection():
@@ -222,6 +229,9 @@ def test_fp8_weight_only_per_tensor_scale_mlp_up_projection():
     assert_no_regression(dx[rows].cpu(), linear.wo_dgrad(dy[rows], q, scale), truth_dx, "e4m3 per-tensor dgrad")
     assert rel_l2(dx[rows].cpu(), truth_dx) <= 4e-3
     assert torch.equal(native.wo_gemm_dgrad(dyg[perm].contiguous(), qg, sg, 0), dx[perm])
+    for cfg in range(1, n_configs()):
+        assert torch.equal(native.wo_gemm_fwd(xg, qg, sg, bg, cfg), y), f"forward cfg{cfg}"
+        assert torch.equal(native.wo_gemm_dgrad(dyg, qg, sg, cfg), dx), f"input gradient cfg{cfg}"
 
 
 def test_argument_errors():
