@@ -18,7 +18,8 @@ CSRC = PKG / "csrc"
 OUT_DIR = PKG / "_lib"
 LIB = OUT_DIR / "libkm_kernels.so"
 HOST_LIB = OUT_DIR / "libkm_hostcheck.so"
-SOURCES = ("km_api.hip", "km_quant.hip", "km_gemm_fp8.hip", "km_gemm_fp8_w32.hip", "km_gemm_blocks.hip", "km_gemm_fused.hip", "km_wo_gemm.hip", "km_wo_dgrad.hip", "km_wo_fwd_bf16.hip", "km_wo_fwd_f16.hip", "km_wo_dgrad_bf16.hip", "km_wo_dgrad_f16.hip", "km_hadamard.hip")
+SOURCES = ("km_api.hip", "km_quant.hip", "km_gemm_fp8.hip", "km_gemm_fp8_w32.hip", "km_gemm_blocks.hip", "km_gemm_fused.hip", "km_wo_gemm.hip", "km_wo_dgrad.hip", "km_wo_fwd_bf16.hip", "km_wo_fwd_f16.hip", "km_wo_dgrad_bf16_i8.hip", "km_wo_dgrad_bf16_e4m3.hip", "km_wo_dgrad_bf16_e4m3b.hip",
+           "km_wo_dgrad_f16_i8.hip", "km_wo_dgrad_f16_e4m3.hip", "km_wo_dgrad_f16_e4m3b.hip", "km_hadamard.hip")
 ARCH = "gfx950"
 # packed fp32 instructions are switched off for every device translation unit
 DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -48,8 +49,15 @@ def build(verbose: bool = True) -> Path:
     OUT_DIR.mkdir(exist_ok=True)
     srcs = [CSRC / s for s in SOURCES if (CSRC / s).exists()]
     objs = [OUT_DIR / (s.stem + ".o") for s in srcs]
-    # the slowest files first: the weight-only tile kernels take minutes each
-    order = sorted(range(len(srcs)), key=lambda i: not srcs[i].name.startswith("km_wo_"))
+    # the slowest files first (each takes minutes): the fp8 GEMM, the weight-only forward kernels,
+    # then the parts of the weight-only input gradient
+    def weight(name: str) -> int:
+        for rank, prefix in enumerate(("km_gemm_fp8.", "km_wo_fwd_", "km_wo_dgrad_bf16_e4m3.", "km_wo_dgrad_f16_e4m3.", "km_wo_dgrad_")):
+            if name.startswith(prefix):
+                return rank
+        return 9
+
+    order = sorted(range(len(srcs)), key=lambda i: weight(srcs[i].name))
     srcs, objs = [srcs[i] for i in order], [objs[i] for i in order]
     with ThreadPoolExecutor(max_workers=min(os.cpu_count() or 4, 12, len(srcs))) as pool:
         list(pool.map(lambda p: _compile(*p), zip(srcs, objs)))

@@ -1,6 +1,6 @@
 // Input gradient of int8 / e4m3 weight-only bases and of fp8 compute bases without a transposed
 // copy, over the codes as they are stored: dx[M,K] = dy[M,N] @ round16(q[N,K] * scale(n,k)). The
-// tiled kernel (km_wo_kernel.h, mode kWoDgradN; built in km_wo_dgrad_bf16.hip and km_wo_dgrad_f16.hip) transposes 8 x 4 bytes of codes in registers on
+// tiled kernel (km_wo_kernel.h, mode kWoDgradN; built in km_wo_dgrad_{bf16,f16}_{i8,e4m3,e4m3b}.hip) transposes 8 x 4 bytes of codes in registers on
 // their way to LDS; shapes it does not take go to a one-thread-per-element kernel.
 #include "km_gemm_common.h"
 #include "km_wo_tiles.h"

@@ -1,5 +1,5 @@
 // Launchers of the tiled weight-only kernels. Each activation type and direction is its own
-// translation unit (km_wo_fwd_bf16.hip, km_wo_fwd_f16.hip, km_wo_dgrad_bf16.hip, km_wo_dgrad_f16.hip):
+// translation unit or several (km_wo_fwd_bf16.hip, km_wo_fwd_f16.hip, km_wo_dgrad_{bf16,f16}_{i8,e4m3,e4m3b}.hip):
 // the kernels take long to compile and build side by side.
 #pragma once
 #include <hip/hip_runtime.h>
@@ -19,10 +19,21 @@ int wo_tiles_fwd(int q_format, int config, const void* a, const void* q, const f
 template <int DT>
 int wo_tiles_dgrad_t(int q_format, int config, const void* a, const void* q_t, const float* scale, void* c, int M, int NO, int KC,
                      hipStream_t st);
-// dx [M, K] = dy [M, N] @ round16(q [N, K] * scale(n, k)) over the codes as stored
+// dx [M, K] = dy [M, N] @ round16(q [N, K] * scale(n, k)) over the codes as stored. The kernels
+// of one activation type are spread over three translation units (int8 codes; e4m3 codes with a
+// scale per row or per tensor; e4m3 codes with E8M0 or 128 x 128 block scales): each `part` is
+// defined in one of km_wo_dgrad_{bf16,f16}_{i8,e4m3,e4m3b}.hip.
+enum { kWoPartI8 = 0, kWoPartE4m3Rows = 1, kWoPartE4m3Blocks = 2 };
+template <int DT, int PART>
+int wo_tiles_dgrad_n_part(int scale_kind, int config, const void* dy, const void* q, const void* scale, int scale_ld, void* dx, int M,
+                          int N, int K, hipStream_t st);
 template <int DT>
-int wo_tiles_dgrad_n(int q_format, int scale_kind, int config, const void* dy, const void* q, const void* scale, int scale_ld, void* dx,
-                     int M, int N, int K, hipStream_t st);
+inline int wo_tiles_dgrad_n(int q_format, int scale_kind, int config, const void* dy, const void* q, const void* scale, int scale_ld,
+                            void* dx, int M, int N, int K, hipStream_t st) {
+  if (q_format == KM_Q_INT8) return wo_tiles_dgrad_n_part<DT, kWoPartI8>(scale_kind, config, dy, q, scale, scale_ld, dx, M, N, K, st);
+  if (scale_kind == KM_WSCALE_ROWS) return wo_tiles_dgrad_n_part<DT, kWoPartE4m3Rows>(scale_kind, config, dy, q, scale, scale_ld, dx, M, N, K, st);
+  return wo_tiles_dgrad_n_part<DT, kWoPartE4m3Blocks>(scale_kind, config, dy, q, scale, scale_ld, dx, M, N, K, st);
+}
 
 // argument checks shared by the entry points
 int check_wo_args(const char* who, const void* a, const void* q, const void* scale, void* c, int64_t M, int64_t N, int64_t K,
