@@ -223,6 +223,10 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
   int wscale[2][WS], xscale[2][XS];
   uint32_t wraw[WS], xraw[XS];
   uint64_t wraw64 = 0, xraw64 = 0;  // packed layout: the 8 scale bytes of a lane
+  // A 96-row wavefront (192-row tiles) may start 64 or 96 rows into a 128-row scale block: its
+  // tiles then continue in the next block, whose 8 bytes are fetched as well.
+  constexpr bool kWStraddle = MX && SCALE_KM && WTN % 64 != 0, kXStraddle = MX && SCALE_KM && WTM % 64 != 0;
+  uint64_t wraw64b = 0, xraw64b = 0;
 
   // one 4 KiB pass (32 rows) of a slab: each wavefront moves 1 KiB with one instruction
   // LDS buffers are named by their LDS byte address (uniform 32-bit values): the B buffers of the
@@ -268,6 +272,9 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
       if constexpr (SCALE_KM) {
         wraw64 = hidden_load_b64(wr, ws_off[0], wso);
         xraw64 = hidden_load_b64(xr, xs_off[0], xso);
+        // the next 128-row block of the same step, clamped to the last one
+        if constexpr (kWStraddle) wraw64b = hidden_load_b64(wr, ws_off[0], __builtin_amdgcn_readfirstlane(ks * ws_step + min(wbase + 512, (rbn - 1) * 512)));
+        if constexpr (kXStraddle) xraw64b = hidden_load_b64(xr, xs_off[0], __builtin_amdgcn_readfirstlane(ks * xs_step + min(xbase + 512, (rbm - 1) * 512)));
       } else {
 #pragma unroll
         for (int t = 0; t < TN; ++t)
@@ -289,8 +296,10 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
 #pragma unroll
       for (int t = 0; t < XS; ++t) xscale[P][t] = (int)(0x7F7F7F7Fu & live);
     } else if constexpr (SCALE_KM) {
-      const uint64_t wv = wraw64 >> wsel;
-      const uint64_t xv = xraw64 >> xsel;
+      uint64_t wv = wraw64 >> wsel;
+      uint64_t xv = xraw64 >> xsel;
+      if constexpr (kWStraddle) wv |= wsel ? wraw64b << (64 - wsel) : 0;
+      if constexpr (kXStraddle) xv |= xsel ? xraw64b << (64 - xsel) : 0;
       wscale[P][0] = (int)((uint32_t)wv & live); wscale[P][1] = (int)((uint32_t)(wv >> 32) & live);
       xscale[P][0] = (int)((uint32_t)xv & live); xscale[P][1] = (int)((uint32_t)(xv >> 32) & live);
     } else {
@@ -540,6 +549,7 @@ static const GemmConfig kGemmConfigs[] = {
     {64, 128, 2, 16},
     {256, 256, 3, 16},
     {256, 256, 2, 32},
+    {256, 192, 2, 16},
 };
 constexpr int kNumGemmConfigs = sizeof(kGemmConfigs) / sizeof(kGemmConfigs[0]);
 
@@ -601,6 +611,9 @@ static int dispatch_config(int config, const void* a, const void* as, const void
       // the int8 MFMA has no 64-deep 32 x 32 form in this pipeline: int8 runs configuration 0 here
       if constexpr (I8) return launch_gemm<256, 256, MX, SCALE_KM, OUT, false, I8>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
       else return gemm_w32(MX, SCALE_KM, OUT, a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
+    // 192 columns: whole waves of tiles for widths like 12288 at short M (8 x 64 = 512 tiles at
+    // M = 2048 where 256-column tiles make 384, one and a half waves)
+    case 7: return launch_gemm<256, 192, MX, SCALE_KM, OUT, false, I8>(a, as, b, bs, sa, sb, bias, c, M, N, K, scale_vectors, st);
   }
   return km_fail(KM_ERR_ARG, "km_gemm: unknown config");
 }
