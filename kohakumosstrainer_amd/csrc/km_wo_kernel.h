@@ -383,8 +383,14 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
     } else if constexpr (NAT && SK == KM_WSCALE_ROWS) {
       const float* scale = static_cast<const float*>(scale_ptr);
       const int n = min(s * 32 + 8 * wave, KC - 8);  // wavefront-uniform
+      // a pointer walked by the stride: one 64-bit multiply per step, not one per load (no branch on
+      // the stride: a wait for the scalar loads would land in the middle of the step)
+      const float* p = scale + (size_t)n * scale_ld;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) sc[set][i] = scale[(size_t)(n + i) * scale_ld];
+      for (int i = 0; i < 8; ++i) {
+        sc[set][i] = *p;
+        p += scale_ld;
+      }
     }
   };
   auto load_slab = [&](int set, int s) __attribute__((always_inline)) {
