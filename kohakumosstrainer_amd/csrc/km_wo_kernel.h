@@ -187,18 +187,13 @@ __device__ __forceinline__ uint32_t widen_pair(uint32_t w, int pair, float s0, f
   }
 }
 
-// The 8 x 4 byte transposition in single instructions. Stage one, p = 4 h + i: rows 4h .. 4h+3 of
-// d, i = 0: columns 0,1 of rows 0,1; 1: columns 2,3 of rows 0,1; 2, 3: the same of rows 2,3.
-__device__ __forceinline__ uint32_t transpose_stage1(const uint32_t (&d)[8], int p) {
+// Half of an 8 x 4 byte transposition is all the widening needs: a dword of two values holds one
+// column of rows 2d, 2d+1, and a byte permute of two row dwords gives two such pairs. p = 4 h + i:
+// rows 4h .. 4h+3 of d, i = 0: columns 0,1 of rows 0,1 (bytes r0c0 r1c0 r0c1 r1c1); 1: columns 2,3 of
+// rows 0,1; 2, 3: the same of rows 2,3.
+__device__ __forceinline__ uint32_t pair_rows(const uint32_t (&d)[8], int p) {
   const uint32_t* r = d + 4 * (p >> 2) + 2 * ((p >> 1) & 1);
   return __builtin_amdgcn_perm(r[1], r[0], (p & 1) ? 0x07030602u : 0x05010400u);
-}
-// Stage two, p = 4 h + j: column j of rows 4h .. 4h+3 from the stage-one words t[4h .. 4h+3]
-__device__ __forceinline__ uint32_t transpose_stage2(const uint32_t (&t)[8], int p) {
-  const uint32_t* r = t + 4 * (p >> 2);
-  const int j = p & 3;
-  // columns 0,1 come from words 0 (rows 0,1) and 2 (rows 2,3); columns 2,3 from words 1 and 3
-  return __builtin_amdgcn_perm(r[2 + (j >> 1)], r[j >> 1], (j & 1) ? 0x07060302u : 0x05040100u);
 }
 
 // how the codes are laid out and scaled
@@ -229,6 +224,13 @@ __device__ __forceinline__ uint64_t loop_load_b64(const v4i& rsrc, int voffset) 
 __device__ __forceinline__ uint32_t loop_load_b32(const v4i& rsrc, int voffset) {
   uint32_t v;
   asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "=v"(v) : "v"(voffset), "s"(rsrc) : "memory");
+  return v;
+}
+typedef int v8i __attribute__((ext_vector_type(8)));
+// scalar load of eight dwords at a wavefront-uniform byte offset; past the descriptor's size reads as zero
+__device__ __forceinline__ v8i loop_sload_x8(const v4i& rsrc, int soffset) {
+  v8i v;
+  asm volatile("s_buffer_load_dwordx8 %0, %1, %2" : "=s"(v) : "s"(rsrc), "s"(soffset) : "memory");
   return v;
 }
 __device__ __forceinline__ uint32_t loop_load_u8(const v4i& rsrc, int voffset) {
@@ -315,6 +317,15 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
 #pragma unroll
     for (int i = 0; i < 8; ++i) sc[b][i] = 1.f;
 
+  // row scales of codes as stored: eight per slab and wavefront, wavefront-uniform
+  constexpr bool kRowScalars = NAT && SK == KM_WSCALE_ROWS;
+  v8i scr[2] = {};
+  v4i row_scale_rsrc = v4i{0, 0, 0, 0};
+  int tensor_scale_bits = 0;
+  if constexpr (kRowScalars) {
+    row_scale_rsrc = raw_rsrc(scale_ptr, scale_ld ? (uint32_t)KC * 4u : 4u);
+    tensor_scale_bits = __builtin_amdgcn_readfirstlane(*static_cast<const int*>(scale_ptr));
+  }
   v4i scale_rsrc = v4i{0, 0, 0, 0};
   if constexpr (NS > 0) {
     const int64_t bytes = SK == KM_WSCALE_E8M0 ? (int64_t)KC * scale_ld : (int64_t)((KC + 127) >> 7) * scale_ld * 4;
@@ -336,24 +347,40 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   auto dma_a_pass = [&](int stage, int a_off, int i) __attribute__((always_inline)) {
     loop_dma_b128(a_rsrc, lds_offset(a_ring) + stage * A_STAGE + (i * 4 + wave) * 1024, a_off + i * (64 * 2) * KC, 0);
   };
+  // K-contiguous codes: one per-lane offset per slab, as for A
   auto q_offset = [&](int s) __attribute__((always_inline)) {
-    if constexpr (!NAT) {
+    if constexpr (NAT) return 0;
+    else {
       const int col = s * 32 + q_chunk * 8;
       return opaque(col < KC ? q_row * KC + col : kOob);
-    } else {
-      // rows n .. n + 7 of q, this thread's four columns; the group is whole (KC % 8 == 0)
-      const int n = s * 32 + 8 * wave;
-      return opaque(n < KC && nat_live ? n * NO + 4 * col4 : kOob);
     }
   };
-  // piece i of the code loads of a slab into register set `set`
+  // Codes as stored: the descriptor of slab s starts at row 32 s of q and ends where q ends, so the
+  // offsets of a lane's eight rows (n = 32 s + 8 wave + i, four columns) do not depend on s, rows
+  // past the end stay out of range and the walk from slab to slab is scalar arithmetic.
+  int q_voff[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) q_voff[i] = NAT ? opaque(nat_live ? (8 * wave + i) * NO + 4 * col4 : kOob) : 0;
+  const int q_slab_bytes = 32 * NO;
+  const uint64_t q_first = (uint64_t)reinterpret_cast<uintptr_t>(Q) + (uint64_t)q_skip;
+  int q_walk_lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)q_first);
+  int q_walk_hi = __builtin_amdgcn_readfirstlane((int)((uint32_t)(q_first >> 32) & 0xFFFFu));
+  int q_walk_left = __builtin_amdgcn_readfirstlane((int)min((int64_t)NO * KC - q_skip, (int64_t)0x7FFFFFFF));
+  auto q_walk_rsrc = [&]() __attribute__((always_inline)) { return v4i{q_walk_lo, q_walk_hi, max(q_walk_left, 0), 0x00020000}; };
+  auto q_walk_advance = [&]() __attribute__((always_inline)) {
+    // the bytes left go negative past the end (by at most 127 rows: no wrap) and are clamped above
+    asm volatile("s_add_u32 %0, %0, %3\n\ts_addc_u32 %1, %1, 0\n\ts_sub_i32 %2, %2, %3"
+                 : "+s"(q_walk_lo), "+s"(q_walk_hi), "+s"(q_walk_left) : "s"(q_slab_bytes) : "scc");
+  };
+  // piece i of the code loads of a slab into register set `set` (codes as stored: of the slab the
+  // walking descriptor stands at)
   auto load_code_piece = [&](int set, int q_off, int i) __attribute__((always_inline)) {
     if constexpr (!NAT) {
       const uint64_t v = loop_load_b64(q_rsrc, q_off + i * 64 * KC);
       raw[set][2 * i] = (uint32_t)v;
       raw[set][2 * i + 1] = (uint32_t)(v >> 32);
     } else {
-      raw[set][i] = loop_load_b32(q_rsrc, q_off + i * NO);
+      raw[set][i] = loop_load_b32(q_walk_rsrc(), q_voff[i]);
     }
   };
   // Scales of slab s. Rows and columns past the end are clamped: their codes are zeros or belong
@@ -380,17 +407,26 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
       const float4 lo = *reinterpret_cast<const float4*>(scale + col), hi = *reinterpret_cast<const float4*>(scale + col + 4);
       sc[set][0] = lo.x; sc[set][1] = lo.y; sc[set][2] = lo.z; sc[set][3] = lo.w;
       sc[set][4] = hi.x; sc[set][5] = hi.y; sc[set][6] = hi.z; sc[set][7] = hi.w;
-    } else if constexpr (NAT && SK == KM_WSCALE_ROWS) {
-      const float* scale = static_cast<const float*>(scale_ptr);
+    } else if constexpr (kRowScalars) {
+      // eight consecutive scales in one range-checked scalar load (with one scale for the whole
+      // tensor every offset but 0 is out of range and reads as zero: select_scales ignores them)
       const int n = min(s * 32 + 8 * wave, KC - 8);  // wavefront-uniform
-      // a pointer walked by the stride: one 64-bit multiply per step, not one per load (no branch on
-      // the stride: a wait for the scalar loads would land in the middle of the step)
-      const float* p = scale + (size_t)n * scale_ld;
+      scr[set] = loop_sload_x8(row_scale_rsrc, n * 4);
+    }
+  };
+  // The scalar load is an opaque statement: its registers are read here, one step-end wait later.
+  auto select_scales = [&](int set) __attribute__((always_inline)) {
+    if constexpr (kRowScalars) {
+      int r[8];
+      asm volatile("s_cmp_lg_u32 %9, 0\n\ts_cselect_b32 %0, %10, %8\n\ts_cselect_b32 %1, %11, %8\n\ts_cselect_b32 %2, %12, %8\n\t"
+                   "s_cselect_b32 %3, %13, %8\n\ts_cselect_b32 %4, %14, %8\n\ts_cselect_b32 %5, %15, %8\n\t"
+                   "s_cselect_b32 %6, %16, %8\n\ts_cselect_b32 %7, %17, %8"
+                   : "=&s"(r[0]), "=&s"(r[1]), "=&s"(r[2]), "=&s"(r[3]), "=&s"(r[4]), "=&s"(r[5]), "=&s"(r[6]), "=&s"(r[7])
+                   : "s"(tensor_scale_bits), "s"(scale_ld), "s"(scr[set][0]), "s"(scr[set][1]), "s"(scr[set][2]), "s"(scr[set][3]),
+                     "s"(scr[set][4]), "s"(scr[set][5]), "s"(scr[set][6]), "s"(scr[set][7])
+                   : "scc");
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        sc[set][i] = *p;
-        p += scale_ld;
-      }
+      for (int i = 0; i < 8; ++i) sc[set][i] = bits_f32((uint32_t)r[i]);
     }
   };
   auto load_slab = [&](int set, int s) __attribute__((always_inline)) {
@@ -400,6 +436,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
     for (int i = 0; i < NS; ++i) load_scale_piece(set, s_off, i);
 #pragma unroll
     for (int i = 0; i < NQ; ++i) load_code_piece(set, q_off, i);
+    if constexpr (NAT) q_walk_advance();  // slabs are requested in order: 0 .. 3 here, s + 4 in step s
   };
   auto dma_a = [&](int stage, int s) __attribute__((always_inline)) {
     const int a_off = a_offset(s);
@@ -407,15 +444,12 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
     for (int i = 0; i < A_LD; ++i) dma_a_pass(stage, a_off, i);
   };
   // The widen-and-store work of a slab in single-instruction pieces, so that each can ride behind
-  // one MFMA. Codes as stored: 8 + 8 byte permutes turn the eight dwords (n, 4 k) into four
-  // (k, 8 n) runs `tq`. Then dword d of unit c (two values of the activation type) comes from one
-  // byte pair, and unit c (four dwords) is one 16-byte LDS write.
-  uint32_t t1[8], tq[8], w16[UNITS][4];
-  auto transpose_piece = [&](int set, int p) __attribute__((always_inline)) {  // p < 16
-    if constexpr (NAT) {
-      if (p < 8) t1[p] = transpose_stage1(raw[set], p);
-      else tq[p - 8] = transpose_stage2(t1, p - 8);  // tq[4 h + j]: rows 4h .. 4h+3 of column j
-    }
+  // one MFMA. Codes as stored: eight byte permutes turn the eight dwords (n, 4 k) into words of two
+  // byte pairs (k, rows 2d and 2d+1) `t1`. Then dword d of unit c (two values of the activation
+  // type) comes from one byte pair, and unit c (four dwords) is one 16-byte LDS write.
+  uint32_t t1[8], w16[UNITS][4];
+  auto transpose_piece = [&](int set, int p) __attribute__((always_inline)) {  // p < 8
+    if constexpr (NAT) t1[p] = pair_rows(raw[set], p);
   };
   auto widen_piece = [&](int set, int c, int d) __attribute__((always_inline)) {
     if constexpr (!NAT) {
@@ -425,7 +459,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
       if constexpr (SK == KM_WSCALE_ROWS) { s0 = sc[set][2 * d]; s1 = sc[set][2 * d + 1]; }
       else if constexpr (SK == KM_WSCALE_E8M0) { s0 = bits_f32(sraw[set][2 * d] << 23); s1 = bits_f32(sraw[set][2 * d + 1] << 23); }
       else { s0 = s1 = bits_f32(sraw[set][0]); }
-      w16[c][d] = widen_pair<DT, QF, true>(tq[4 * (d >> 1) + c], d & 1, s0, s1);  // column c, rows 2d, 2d+1
+      w16[c][d] = widen_pair<DT, QF, true>(t1[2 * d + (c >> 1)], c & 1, s0, s1);  // column c, rows 2d, 2d+1
     }
   };
   auto store_unit = [&](int stage, int c) __attribute__((always_inline)) {
@@ -435,8 +469,9 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
     else if (nat_live) *reinterpret_cast<uint4*>(slab + slab32_offset(nat_row0 + c * nat_stride, wave)) = v;
   };
   auto commit_all = [&](int set, int stage) __attribute__((always_inline)) {
+    select_scales(set);
 #pragma unroll
-    for (int p = 0; p < 16; ++p) transpose_piece(set, p);
+    for (int p = 0; p < 8; ++p) transpose_piece(set, p);
 #pragma unroll
     for (int c = 0; c < UNITS; ++c) {
 #pragma unroll
@@ -483,6 +518,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
       constexpr int q = decltype(q_tag)::value;
       constexpr int t = q / TM, j = q % TM;
       mfma16<DT>(acc[t][j], wf[par][t], xf[par][j]);
+      if constexpr (q == 0) select_scales(par);
       static_for<NR>([&](auto r_tag) __attribute__((always_inline)) {
         constexpr int r = decltype(r_tag)::value;
         if constexpr (q == at(r, NR, 0, S / 2)) read_fragment(par ^ 1, (u + 1) & 3, r);
@@ -491,9 +527,9 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
         constexpr int i = decltype(i_tag)::value;
         if constexpr (q == at(i, A_LD, 0, S / 2)) dma_a_pass((u + 3) & 3, a_off, i);
       });
-      static_for<16>([&](auto p_tag) __attribute__((always_inline)) {
+      static_for<8>([&](auto p_tag) __attribute__((always_inline)) {
         constexpr int pp = decltype(p_tag)::value;
-        if constexpr (NAT && q == at(pp, 16, S / 4, S / 2)) transpose_piece(par, pp);
+        if constexpr (NAT && q == at(pp, 8, S / 4, S / 2)) transpose_piece(par, pp);
       });
       static_for<4 * UNITS>([&](auto p_tag) __attribute__((always_inline)) {
         constexpr int pp = decltype(p_tag)::value;
@@ -510,7 +546,8 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
       if constexpr (q == L0) load_scalar_scales(par, s + 4);
       // the offsets of the next step's loads, a few instructions each
       if constexpr (q == at(0, 3, S / 2, S)) next_a_off = a_offset(s + 4);
-      if constexpr (q == at(1, 3, S / 2, S)) next_q_off = q_offset(s + 5);
+      if constexpr (q == at(1, 3, S / 2, S) && !NAT) next_q_off = q_offset(s + 5);
+      if constexpr (q == S - 1 && NAT) q_walk_advance();
       if constexpr (q == at(2, 3, S / 2, S) && NS > 0) next_s_off = scale_offset(s + 5);
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -573,6 +610,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
     for (int i = 0; i < (NAT ? 8 : 2 * UNITS); ++i) asm volatile("" ::"v"(raw[b][i]));
 #pragma unroll
     for (int i = 0; i < (NS ? NS : 1); ++i) asm volatile("" ::"v"(sraw[b][i]));
+    if constexpr (kRowScalars) asm volatile("" ::"s"(scr[b]));
   }
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
