@@ -85,15 +85,16 @@ __global__ __launch_bounds__(256) void transpose_bytes(const uint8_t* __restrict
 }
 
 struct WoConfig {
-  int bm, bn;
+  int bm, bn, tail_bm;
 };
-static const WoConfig kWoConfigs[] = {{256, 256}, {128, 256}, {256, 128}, {128, 128}, {64, 128}, {256, 192}};
+static const WoConfig kWoConfigs[] = {{256, 256, 0}, {128, 256, 0}, {256, 128, 0}, {128, 128, 0}, {64, 128, 0}, {256, 192, 0}, {256, 256, 128}};
 static_assert(sizeof(kWoConfigs) / sizeof(kWoConfigs[0]) == kNumWoConfigs, "one row per case of launch_config");
 
 int wo_num_configs() { return kNumWoConfigs; }
 int wo_config_desc(int config, char* buf, int len) {
   if (config < 0 || config >= kNumWoConfigs) return km_fail(KM_ERR_ARG, "config out of range");
-  snprintf(buf, len, "bm=%d,bn=%d,bk=64,waves=4", kWoConfigs[config].bm, kWoConfigs[config].bn);
+  // tail_bm: rows of the tiles that cover what whole rounds of bm x bn tiles leave over (0: none)
+  snprintf(buf, len, "bm=%d,bn=%d,bk=64,waves=4,tail_bm=%d", kWoConfigs[config].bm, kWoConfigs[config].bn, kWoConfigs[config].tail_bm);
   return KM_OK;
 }
 

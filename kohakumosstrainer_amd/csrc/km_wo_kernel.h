@@ -226,10 +226,10 @@ __device__ __forceinline__ uint32_t loop_load_b32(const v4i& rsrc, int voffset) 
   asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "=v"(v) : "v"(voffset), "s"(rsrc) : "memory");
   return v;
 }
-typedef int v8i __attribute__((ext_vector_type(8)));
-// scalar load of eight dwords at a wavefront-uniform byte offset; past the descriptor's size reads as zero
-__device__ __forceinline__ v8i loop_sload_x8(const v4i& rsrc, int soffset) {
-  v8i v;
+typedef uint64_t v4u64 __attribute__((ext_vector_type(4)));
+// scalar load of eight dwords (as four pairs) at a wavefront-uniform byte offset; past the descriptor's size reads as zero
+__device__ __forceinline__ v4u64 loop_sload_x8(const v4i& rsrc, int soffset) {
+  v4u64 v;
   asm volatile("s_buffer_load_dwordx8 %0, %1, %2" : "=s"(v) : "s"(rsrc), "s"(soffset) : "memory");
   return v;
 }
@@ -248,7 +248,8 @@ template <int BM, int BN, int DT, int QF, int MODE, int SK>
 __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict__ A, const uint8_t* __restrict__ Q,
                                                       const void* __restrict__ scale_ptr, int scale_ld,
                                                       const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int NO,
-                                                      int KC) {
+                                                      int KC, int tn_first, int tn_count) {
+  // the grid covers tile columns tn_first .. tn_first + tn_count - 1 of the output
   constexpr int WTM = BM / 2, WTN = BN / 2;
   constexpr int TM = WTM / 16, TN = WTN / 16;
   constexpr int STAGES = 4;
@@ -266,8 +267,8 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   __shared__ __attribute__((aligned(1024))) uint8_t b_ring[STAGES * B_STAGE];
 
   int tile_m, tile_n;
-  tile_of(blockIdx.x, (M + BM - 1) / BM, (NO + BN - 1) / BN, tile_m, tile_n);
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  tile_of(blockIdx.x, (M + BM - 1) / BM, tn_count, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = (tn_first + tile_n) * BN;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = (wave >> 1) * WTM, wn = (wave & 1) * WTN;
@@ -319,12 +320,13 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
 
   // row scales of codes as stored: eight per slab and wavefront, wavefront-uniform
   constexpr bool kRowScalars = NAT && SK == KM_WSCALE_ROWS;
-  v8i scr[2] = {};
+  v4u64 scr[2] = {};
   v4i row_scale_rsrc = v4i{0, 0, 0, 0};
-  int tensor_scale_bits = 0;
+  uint64_t tensor_scale_twice = 0;  // zero with row scales
   if constexpr (kRowScalars) {
     row_scale_rsrc = raw_rsrc(scale_ptr, scale_ld ? (uint32_t)KC * 4u : 4u);
-    tensor_scale_bits = __builtin_amdgcn_readfirstlane(*static_cast<const int*>(scale_ptr));
+    const uint32_t bits = scale_ld ? 0u : (uint32_t)__builtin_amdgcn_readfirstlane(*static_cast<const int*>(scale_ptr));
+    tensor_scale_twice = ((uint64_t)bits << 32) | bits;
   }
   v4i scale_rsrc = v4i{0, 0, 0, 0};
   if constexpr (NS > 0) {
@@ -409,24 +411,23 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
       sc[set][4] = hi.x; sc[set][5] = hi.y; sc[set][6] = hi.z; sc[set][7] = hi.w;
     } else if constexpr (kRowScalars) {
       // eight consecutive scales in one range-checked scalar load (with one scale for the whole
-      // tensor every offset but 0 is out of range and reads as zero: select_scales ignores them)
+      // tensor every offset but 0 is out of range and reads as zero)
       const int n = min(s * 32 + 8 * wave, KC - 8);  // wavefront-uniform
       scr[set] = loop_sload_x8(row_scale_rsrc, n * 4);
     }
   };
   // The scalar load is an opaque statement: its registers are read here, one step-end wait later.
+  // Row scales pass through; of a per-tensor scale the load brought zeros (or the scale itself, at
+  // offset 0), and the scale is ORed over every one, two at a time.
   auto select_scales = [&](int set) __attribute__((always_inline)) {
     if constexpr (kRowScalars) {
-      int r[8];
-      asm volatile("s_cmp_lg_u32 %9, 0\n\ts_cselect_b32 %0, %10, %8\n\ts_cselect_b32 %1, %11, %8\n\ts_cselect_b32 %2, %12, %8\n\t"
-                   "s_cselect_b32 %3, %13, %8\n\ts_cselect_b32 %4, %14, %8\n\ts_cselect_b32 %5, %15, %8\n\t"
-                   "s_cselect_b32 %6, %16, %8\n\ts_cselect_b32 %7, %17, %8"
-                   : "=&s"(r[0]), "=&s"(r[1]), "=&s"(r[2]), "=&s"(r[3]), "=&s"(r[4]), "=&s"(r[5]), "=&s"(r[6]), "=&s"(r[7])
-                   : "s"(tensor_scale_bits), "s"(scale_ld), "s"(scr[set][0]), "s"(scr[set][1]), "s"(scr[set][2]), "s"(scr[set][3]),
-                     "s"(scr[set][4]), "s"(scr[set][5]), "s"(scr[set][6]), "s"(scr[set][7])
+      uint64_t r[4];
+      asm volatile("s_or_b64 %0, %4, %8\n\ts_or_b64 %1, %5, %8\n\ts_or_b64 %2, %6, %8\n\ts_or_b64 %3, %7, %8"
+                   : "=&s"(r[0]), "=&s"(r[1]), "=&s"(r[2]), "=&s"(r[3])
+                   : "s"(scr[set][0]), "s"(scr[set][1]), "s"(scr[set][2]), "s"(scr[set][3]), "s"(tensor_scale_twice)
                    : "scc");
 #pragma unroll
-      for (int i = 0; i < 8; ++i) sc[set][i] = bits_f32((uint32_t)r[i]);
+      for (int i = 0; i < 8; ++i) sc[set][i] = bits_f32((uint32_t)(r[i >> 1] >> (32 * (i & 1))));
     }
   };
   auto load_slab = [&](int set, int s) __attribute__((always_inline)) {
@@ -449,7 +450,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   // type) comes from one byte pair, and unit c (four dwords) is one 16-byte LDS write.
   uint32_t t1[8], w16[UNITS][4];
   auto transpose_piece = [&](int set, int p) __attribute__((always_inline)) {  // p < 8
-    if constexpr (NAT) t1[p] = pair_rows(raw[set], p);
+    if constexpr (NAT && QF != KM_Q_INT8) t1[p] = pair_rows(raw[set], p);  // an int8 conversion selects its byte by itself
   };
   auto widen_piece = [&](int set, int c, int d) __attribute__((always_inline)) {
     if constexpr (!NAT) {
@@ -459,7 +460,13 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
       if constexpr (SK == KM_WSCALE_ROWS) { s0 = sc[set][2 * d]; s1 = sc[set][2 * d + 1]; }
       else if constexpr (SK == KM_WSCALE_E8M0) { s0 = bits_f32(sraw[set][2 * d] << 23); s1 = bits_f32(sraw[set][2 * d + 1] << 23); }
       else { s0 = s1 = bits_f32(sraw[set][0]); }
-      w16[c][d] = widen_pair<DT, QF, true>(t1[2 * d + (c >> 1)], c & 1, s0, s1);  // column c, rows 2d, 2d+1
+      if constexpr (QF == KM_Q_INT8) {
+        const float f0 = (float)(int)(int8_t)((raw[set][2 * d] >> (8 * c)) & 0xFFu) * s0;
+        const float f1 = (float)(int)(int8_t)((raw[set][2 * d + 1] >> (8 * c)) & 0xFFu) * s1;
+        w16[c][d] = pack2<DT>(f0, f1);
+      } else {
+        w16[c][d] = widen_pair<DT, QF, true>(t1[2 * d + (c >> 1)], c & 1, s0, s1);  // column c, rows 2d, 2d+1
+      }
     }
   };
   auto store_unit = [&](int stage, int c) __attribute__((always_inline)) {
@@ -632,11 +639,22 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
 
 template <int BM, int BN, int DT, int QF, int MODE, int SK>
 inline int launch_wo(const void* a, const void* q, const void* scale, int scale_ld, const void* bias, void* c, int M, int NO,
-                     int KC, hipStream_t st) {
-  const int tiles = ((M + BM - 1) / BM) * ((NO + BN - 1) / BN);
+                     int KC, hipStream_t st, int tn_first = 0, int tn_count = -1) {
+  if (tn_count < 0) tn_count = (NO + BN - 1) / BN - tn_first;  // to the last tile column
+  if (tn_count == 0) return KM_OK;
+  const int tiles = ((M + BM - 1) / BM) * tn_count;
   hipLaunchKernelGGL((wo_gemm_kernel<BM, BN, DT, QF, MODE, SK>), dim3(tiles), dim3(256), 0, st, (const uint16_t*)a,
-                     (const uint8_t*)q, scale, scale_ld, (const uint16_t*)bias, (uint16_t*)c, M, NO, KC);
+                     (const uint8_t*)q, scale, scale_ld, (const uint16_t*)bias, (uint16_t*)c, M, NO, KC, tn_first, tn_count);
   return km_check_launch("km_wo_gemm");
+}
+
+// compute units of the current device (asked once per device; not a stream operation)
+inline int compute_units() {
+  static int cached[64] = {};
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cached[dev] == 0 && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess) cached[dev] = n;
+  return cached[dev];
 }
 
 template <int DT, int QF, int MODE, int SK>
@@ -653,6 +671,19 @@ inline int launch_config(int config, const void* a, const void* q, const void* s
       // output columns: 16 x 16 = 256 tiles against 16 x 12 = 192 at M = 4096, 32 x 16 = 512 against
       // 32 x 12 = 384 at M = 8192)
       return launch_wo<256, 192, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st);
+    case 6: {
+      // 256 x 256 tiles over as many tile columns as fill whole rounds of the card (one tile per
+      // compute unit and round), 128 x 256 tiles over the rest: the last, partly empty round of large
+      // tiles becomes a full round of tiles that take less time (8192 x 3072 outputs: 384 large tiles
+      // are one round and a half, so two; 256 large and 256 half tiles are one round each). Every
+      // output element is the same sum in the same order as in the other configurations.
+      const int tm = (M + 255) / 256, tn = (NO + 255) / 256, cus = compute_units();
+      if (cus <= 0) return km_fail(KM_ERR_LAUNCH, "km_wo_gemm: cannot ask for the number of compute units");
+      const int whole_cols = (tm * tn) % cus == 0 ? tn : (int)(((int64_t)tm * tn / cus) * cus / tm);
+      int rc = launch_wo<256, 256, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st, 0, whole_cols);
+      if (rc == KM_OK) rc = launch_wo<128, 256, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st, whole_cols, tn - whole_cols);
+      return rc;
+    }
   }
   return km_fail(KM_ERR_ARG, "km_wo_gemm: unknown config");
 }

@@ -103,6 +103,29 @@ def test_input_gradient_of_an_fp8_base_without_a_transposed_copy(recipe, dtype, 
     assert torch.equal(back, formats.dequantize(q, scale, recipe, dtype)[:256])
 
 
+@pytest.mark.parametrize("fmt", ("int8", "fp8"))
+def test_two_tile_shapes_in_one_call(fmt):
+    """The configuration with `tail_bm` covers whole rounds of the card with 256 x 256 tiles and the
+    remaining tile columns with 128 x 256 tiles in a second launch. 17 x 17 large tiles are more
+    than the card's compute units and not a multiple of them, rows and columns are ragged, and the
+    columns of the second launch start in the middle of the output: every element must equal the
+    one-shape configuration's bit for bit, forward (bias and scale follow the column window) and
+    input gradient."""
+    mixed = [c["id"] for c in native.configs(native.KERNEL_WO_FWD) if c.get("tail_bm", 0)]
+    assert mixed, "no configuration with a tail"
+    m, wide, deep = 4100, 4200, 264
+    x, q, scale, bias, _ = case(m, wide, deep, fmt, torch.bfloat16, seed=3)  # forward: 4200 output columns
+    y0 = native.wo_gemm_fwd(x.cuda(), q.cuda(), scale.cuda(), bias.cuda(), 0)
+    _, q2, scale2, _, dy = case(m, deep, wide, fmt, torch.bfloat16, seed=4)  # gradient: 4200 input features
+    dx0 = native.wo_gemm_dgrad(dy.cuda(), q2.cuda(), scale2.cuda(), 0)
+    assert rel_l2(y0.cpu(), x.double() @ linear.wo_exact64(q, scale).T + bias.double()) <= 2e-3
+    # the gradient multiplies by the weight rounded to 16 bits: judged next to the eager result
+    assert_no_regression(dx0.cpu(), linear.wo_dgrad(dy, q2, scale2), dy.double() @ linear.wo_exact64(q2, scale2), f"wo dgrad {fmt} 17 x 17 tiles")
+    for cfg in mixed:
+        assert torch.equal(native.wo_gemm_fwd(x.cuda(), q.cuda(), scale.cuda(), bias.cuda(), cfg), y0)
+        assert torch.equal(native.wo_gemm_dgrad(dy.cuda(), q2.cuda(), scale2.cuda(), cfg), dx0)
+
+
 @pytest.mark.parametrize("fmt,recipe", (("int8", "row"), ("fp8", "row"), ("fp8", "mx")))
 @pytest.mark.parametrize("m,n,k", ((37, 100, 50), (130, 96, 66), (16, 64, 1), (5, 0, 64)))
 def test_input_gradient_shapes_off_the_vector_path(fmt, recipe, m, n, k):
