@@ -10,6 +10,7 @@
 
 #include "km_internal.h"
 #include "km_numeric.h"
+#include "km_tile_plan.h"
 
 namespace km {
 
@@ -46,24 +47,6 @@ __device__ __forceinline__ float unpack1<KM_BF16>(uint32_t h) { return bits_f32(
 template <>
 __device__ __forceinline__ float unpack1<KM_F16>(uint32_t h) {
   return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
-}
-
-// Work-group id -> (tile_m, tile_n). Work-groups are dealt round-robin to the 8 XCDs, each
-// with its own L2; first give every XCD a contiguous run of tiles, then walk that run in
-// bands of kGroupM row-tiles so that neighbours in time share A rows and B rows in L2.
-constexpr int kXcds = 8;
-constexpr int kGroupM = 8;
-__device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
-  const int total = tiles_m * tiles_n;
-  const int xcd = pid % kXcds, local = pid / kXcds;
-  const int tall = total / kXcds, rem = total % kXcds;
-  int p = xcd < rem ? xcd * (tall + 1) + local : rem * (tall + 1) + (xcd - rem) * tall + local;
-  const int per_group = kGroupM * tiles_n;
-  const int first_m = (p / per_group) * kGroupM;
-  const int group_m = min(tiles_m - first_m, kGroupM);
-  const int in_group = p % per_group;
-  tm = first_m + in_group % group_m;
-  tn = in_group / group_m;
 }
 
 // compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)

@@ -679,7 +679,7 @@ inline int launch_config(int config, const void* a, const void* q, const void* s
       // output element is the same sum in the same order as in the other configurations.
       const int tm = (M + 255) / 256, tn = (NO + 255) / 256, cus = compute_units();
       if (cus <= 0) return km_fail(KM_ERR_LAUNCH, "km_wo_gemm: cannot ask for the number of compute units");
-      const int whole_cols = (tm * tn) % cus == 0 ? tn : (int)(((int64_t)tm * tn / cus) * cus / tm);
+      const int whole_cols = whole_round_columns(tm, tn, cus);
       int rc = launch_wo<256, 256, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st, 0, whole_cols);
       if (rc == KM_OK) rc = launch_wo<128, 256, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st, whole_cols, tn - whole_cols);
       return rc;

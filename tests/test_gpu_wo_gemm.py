@@ -126,6 +126,32 @@ def test_two_tile_shapes_in_one_call(fmt):
         assert torch.equal(native.wo_gemm_dgrad(dy.cuda(), q2.cuda(), scale2.cuda(), cfg), dx0)
 
 
+def test_two_tile_shapes_under_graph_capture():
+    """Both launches of the two-shape configuration, and its question to the runtime about the
+    number of compute units, inside a captured stream: every replay equals the eager result (inputs
+    refilled between replays, eager work in between)."""
+    mixed = [c["id"] for c in native.configs(native.KERNEL_WO_FWD) if c.get("tail_bm", 0)][0]
+    m, n, k = 4100, 264, 4200
+    _, q, scale, _, dy = case(m, n, k, "fp8", torch.bfloat16, seed=6)
+    dq, dscale, static_dy = q.cuda(), scale.cuda(), dy.cuda()
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        native.wo_gemm_dgrad(static_dy, dq, dscale, 0)  # the library is loaded; the mixed configuration may be new to it
+    torch.cuda.current_stream().wait_stream(stream)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        dx_graph = native.wo_gemm_dgrad(static_dy, dq, dscale, mixed)
+    g = torch.Generator().manual_seed(7)
+    for i in range(3):
+        fresh = (torch.randn(m, n, generator=g) * (i + 1)).to(torch.bfloat16).cuda()
+        static_dy.copy_(fresh)
+        graph.replay()
+        eager = native.wo_gemm_dgrad(fresh, dq, dscale, 0)
+        torch.cuda.synchronize()
+        assert torch.equal(dx_graph, eager), f"replay {i}"
+
+
 @pytest.mark.parametrize("fmt,recipe", (("int8", "row"), ("fp8", "row"), ("fp8", "mx")))
 @pytest.mark.parametrize("m,n,k", ((37, 100, 50), (130, 96, 66), (16, 64, 1), (5, 0, 64)))
 def test_input_gradient_shapes_off_the_vector_path(fmt, recipe, m, n, k):
