@@ -16,8 +16,8 @@ void km_host_mx_biased_many(const float* amax, long n, unsigned char* out) {
   for (long i = 0; i < n; ++i) out[i] = (unsigned char)km::mx_biased_exponent(km::f32_bits(amax[i]) & km::kAbsMask);
 }
 // tile of every work-group id of a tiles_m x tiles_n launch: out[2 pid] = tile_m, out[2 pid + 1] = tile_n
-void km_host_tiles_of(int tiles_m, int tiles_n, int* out) {
-  for (int pid = 0; pid < tiles_m * tiles_n; ++pid) km::tile_of(pid, tiles_m, tiles_n, out[2 * pid], out[2 * pid + 1]);
+void km_host_tiles_of(int tiles_m, int tiles_n, int group_m, int* out) {
+  for (int pid = 0; pid < tiles_m * tiles_n; ++pid) km::tile_of(pid, tiles_m, tiles_n, out[2 * pid], out[2 * pid + 1], group_m);
 }
 int km_host_whole_round_columns(int tiles_m, int tiles_n, int units) { return km::whole_round_columns(tiles_m, tiles_n, units); }
 void km_host_bf16_many(const float* v, long n, unsigned short* out) {

@@ -267,7 +267,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   __shared__ __attribute__((aligned(1024))) uint8_t b_ring[STAGES * B_STAGE];
 
   int tile_m, tile_n;
-  tile_of(blockIdx.x, (M + BM - 1) / BM, tn_count, tile_m, tile_n);
+  tile_of(blockIdx.x, (M + BM - 1) / BM, tn_count, tile_m, tile_n, kGroupMWideA);
   const int m0 = tile_m * BM, n0 = (tn_first + tile_n) * BN;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -17,39 +17,42 @@ XCDS = 8
 @pytest.fixture(scope="module")
 def host():
     lib = ctypes.CDLL(str(km_build.build_hostcheck()))
-    lib.km_host_tiles_of.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.km_host_tiles_of.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
     lib.km_host_tiles_of.restype = None
     lib.km_host_whole_round_columns.argtypes = [ctypes.c_int] * 3
     return lib
 
 
-def tiles_of(lib, tiles_m, tiles_n):
+def tiles_of(lib, tiles_m, tiles_n, group_m):
     out = np.empty((tiles_m * tiles_n, 2), dtype=np.int32)
-    lib.km_host_tiles_of(tiles_m, tiles_n, out.ctypes.data)
+    lib.km_host_tiles_of(tiles_m, tiles_n, group_m, out.ctypes.data)
     return out
+
+
+BANDS = (8, 4)  # tile rows per band: the fp8 / int8 GEMMs, the weight-only GEMMs
 
 
 GRIDS = [(m, n) for m in range(1, 20) for n in range(1, 14)] + [(64, 36), (32, 48), (32, 12), (16, 12), (274, 1), (1, 300), (33, 17)]
 
 
 def test_every_tile_is_computed_exactly_once(host):
-    for tiles_m, tiles_n in GRIDS:
-        t = tiles_of(host, tiles_m, tiles_n)
+    for tiles_m, tiles_n, band in [(m, n, b) for m, n in GRIDS for b in BANDS]:
+        t = tiles_of(host, tiles_m, tiles_n, band)
         assert t[:, 0].min() >= 0 and t[:, 0].max() < tiles_m and t[:, 1].min() >= 0 and t[:, 1].max() < tiles_n
         flat = t[:, 0].astype(np.int64) * tiles_n + t[:, 1]
         assert np.array_equal(np.sort(flat), np.arange(tiles_m * tiles_n)), (tiles_m, tiles_n)
 
 
-def test_an_xcd_walks_a_contiguous_run_in_bands_of_eight_rows(host):
+def test_an_xcd_walks_a_contiguous_run_of_the_band_order(host):
     """Work-group ids go round-robin over the XCDs. The tiles of one XCD, in the order it gets them,
-    must be a contiguous stretch of the band order (bands of eight tile rows, column by column
+    must be a contiguous stretch of the band order (bands of eight or four tile rows, column by column
     within a band, rows fastest), so that neighbours in time share operand rows in that XCD's L2."""
-    for tiles_m, tiles_n in [(64, 36), (32, 12), (33, 17), (5, 3), (8, 8)]:
-        t = tiles_of(host, tiles_m, tiles_n)
+    for tiles_m, tiles_n, band in [(m, n, b) for m, n in [(64, 36), (32, 12), (33, 17), (5, 3), (8, 8)] for b in BANDS]:
+        t = tiles_of(host, tiles_m, tiles_n, band)
         order = {}
         p = 0
-        for first in range(0, tiles_m, 8):
-            rows = min(8, tiles_m - first)
+        for first in range(0, tiles_m, band):
+            rows = min(band, tiles_m - first)
             for tn in range(tiles_n):
                 for r in range(rows):
                     order[(first + r, tn)] = p
