@@ -419,7 +419,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   // The scalar load is an opaque statement: its registers are read here, one step-end wait later.
   // Row scales pass through; of a per-tensor scale the load brought zeros (or the scale itself, at
   // offset 0), and the scale is ORed over every one, two at a time.
-  auto select_scales = [&](int set) __attribute__((always_inline)) {
+  auto merge_scales = [&](int set) __attribute__((always_inline)) {
     if constexpr (kRowScalars) {
       uint64_t r[4];
       asm volatile("s_or_b64 %0, %4, %8\n\ts_or_b64 %1, %5, %8\n\ts_or_b64 %2, %6, %8\n\ts_or_b64 %3, %7, %8"
@@ -476,7 +476,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
     else if (nat_live) *reinterpret_cast<uint4*>(slab + slab32_offset(nat_row0 + c * nat_stride, wave)) = v;
   };
   auto commit_all = [&](int set, int stage) __attribute__((always_inline)) {
-    select_scales(set);
+    merge_scales(set);
 #pragma unroll
     for (int p = 0; p < 8; ++p) transpose_piece(set, p);
 #pragma unroll
@@ -525,7 +525,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
       constexpr int q = decltype(q_tag)::value;
       constexpr int t = q / TM, j = q % TM;
       mfma16<DT>(acc[t][j], wf[par][t], xf[par][j]);
-      if constexpr (q == 0) select_scales(par);
+      if constexpr (q == 0) merge_scales(par);
       static_for<NR>([&](auto r_tag) __attribute__((always_inline)) {
         constexpr int r = decltype(r_tag)::value;
         if constexpr (q == at(r, NR, 0, S / 2)) read_fragment(par ^ 1, (u + 1) & 3, r);
