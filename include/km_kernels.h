@@ -225,8 +225,8 @@ int km_group_hadamard(const void *x, int64_t rows, int64_t cols, int dtype, int 
 /* Tile configurations per kernel, for the host-side tuning table (the reference enumerates its
  * Triton tiles in backends/triton/fp8/linear.py:39-75 and backends/triton/quant.py:132-141).
  * km_config_desc writes "key=value,..." (bm, bn: rows and columns of a work-group's tile; for the
- * weight-only kernels tail_bm > 0 names the rows of the smaller tiles that a second launch puts over
- * the tile columns which whole rounds of the card's compute units leave over). */
+ * weight-only kernels tail=1 means that a second launch puts half-size tiles over the tile columns
+ * which whole rounds of the card's compute units leave over). */
 int km_num_configs(int kernel);
 int km_config_desc(int kernel, int config, char *buf, int len);
 

@@ -85,16 +85,16 @@ __global__ __launch_bounds__(256) void transpose_bytes(const uint8_t* __restrict
 }
 
 struct WoConfig {
-  int bm, bn, tail_bm;
+  int bm, bn, tail;
 };
-static const WoConfig kWoConfigs[] = {{256, 256, 0}, {128, 256, 0}, {256, 128, 0}, {128, 128, 0}, {64, 128, 0}, {256, 192, 0}, {256, 256, 128}};
+static const WoConfig kWoConfigs[] = {{256, 256, 0}, {128, 256, 0}, {256, 128, 0}, {128, 128, 0}, {64, 128, 0}, {256, 192, 0}, {256, 256, 1}};
 static_assert(sizeof(kWoConfigs) / sizeof(kWoConfigs[0]) == kNumWoConfigs, "one row per case of launch_config");
 
 int wo_num_configs() { return kNumWoConfigs; }
 int wo_config_desc(int config, char* buf, int len) {
   if (config < 0 || config >= kNumWoConfigs) return km_fail(KM_ERR_ARG, "config out of range");
-  // tail_bm: rows of the tiles that cover what whole rounds of bm x bn tiles leave over (0: none)
-  snprintf(buf, len, "bm=%d,bn=%d,bk=64,waves=4,tail_bm=%d", kWoConfigs[config].bm, kWoConfigs[config].bn, kWoConfigs[config].tail_bm);
+  // tail=1: half-size tiles (128 x 256 or 256 x 128) cover what whole rounds of bm x bn tiles leave over
+  snprintf(buf, len, "bm=%d,bn=%d,bk=64,waves=4,tail=%d", kWoConfigs[config].bm, kWoConfigs[config].bn, kWoConfigs[config].tail);
   return KM_OK;
 }
 

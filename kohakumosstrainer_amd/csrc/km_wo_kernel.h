@@ -233,6 +233,11 @@ __device__ __forceinline__ v4u64 loop_sload_x8(const v4i& rsrc, int soffset) {
   asm volatile("s_buffer_load_dwordx8 %0, %1, %2" : "=s"(v) : "s"(rsrc), "s"(soffset) : "memory");
   return v;
 }
+__device__ __forceinline__ v4i loop_load_b128(const v4i& rsrc, int voffset) {
+  v4i v;
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(v) : "v"(voffset), "s"(rsrc) : "memory");
+  return v;
+}
 __device__ __forceinline__ uint32_t loop_load_u8(const v4i& rsrc, int voffset) {
   uint32_t v;
   asm volatile("buffer_load_ubyte %0, %1, %2, 0 offen" : "=v"(v) : "v"(voffset), "s"(rsrc) : "memory");
@@ -258,8 +263,14 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   constexpr bool NAT = MODE == kWoDgradN;
   constexpr bool PRESCALE = MODE != kWoFwd;
   constexpr int UNITS = NAT ? 4 : BN / 64;             // 16-byte LDS writes per thread and step
-  constexpr int NQ = NAT ? 8 : UNITS;                  // code loads per thread and step
-  constexpr int NS = !NAT ? 0 : SK == KM_WSCALE_E8M0 ? 8 : SK == KM_WSCALE_BLOCKS ? 1 : 0;  // scale loads through the vector path
+  // Codes as stored, 128 columns, a scale per row: the 32 dwords of a row n keep half a wavefront
+  // busy, so the halves take four rows n each (everything per lane and step halves: loads,
+  // permutes, conversions; a lane writes 8 bytes per column instead of 16).
+  constexpr bool kHalfRows = NAT && BN == 128 && SK == KM_WSCALE_ROWS;
+  constexpr int NROWS = kHalfRows ? 4 : 8;             // rows n per lane (codes as stored)
+  constexpr int DPC = NROWS / 2;                       // dwords of two values per column
+  constexpr int NQ = NAT ? NROWS : UNITS;              // code loads per thread and step
+  constexpr int NS = !NAT ? 0 : SK == KM_WSCALE_E8M0 ? 8 : (SK == KM_WSCALE_BLOCKS || kHalfRows) ? 1 : 0;  // scale loads through the vector path
   constexpr int NV = A_LD + NQ + NS;                   // vector-memory loads issued per step, counted by hand below
   static_assert(!NAT || BN == 256 || BN == 192 || BN == 128, "the transposing load covers 256, 192 or 128 columns");
   static_assert(NV < 48, "vmcnt holds 6 bits");
@@ -293,7 +304,8 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   // of a 128-column tile load nothing and write nothing); wavefront w owns rows n = 8 w .. 8 w + 7
   // of the step's 32, which become chunk w of the slab rows
   constexpr int LPR = BN / 4;
-  const bool nat_live = lane < LPR;
+  const bool nat_live = kHalfRows || lane < LPR;
+  const int row_half = kHalfRows ? lane / LPR : 0;           // rows n = 8 wave + 4 row_half .. + 3
   const int col4 = lane % LPR;                               // columns 4 col4 .. 4 col4 + 3 of the tile
   const int half_w = col4 / (LPR / 2), col_l = col4 % (LPR / 2);
   // slab row of column j: nat_row0 + j * nat_stride. A wavefront's WTN / 4 dwords per row n are laid
@@ -312,18 +324,18 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   // codes and scales in flight, set s & 1 for slab s
   uint32_t raw[2][NAT ? 8 : 2 * UNITS];
   float sc[2][8];
-  uint32_t sraw[2][NS ? NS : 1];
+  uint32_t sraw[2][kHalfRows ? 4 : NS ? NS : 1];
 #pragma unroll
   for (int b = 0; b < 2; ++b)
 #pragma unroll
     for (int i = 0; i < 8; ++i) sc[b][i] = 1.f;
 
   // row scales of codes as stored: eight per slab and wavefront, wavefront-uniform
-  constexpr bool kRowScalars = NAT && SK == KM_WSCALE_ROWS;
+  constexpr bool kRowScalars = NAT && SK == KM_WSCALE_ROWS && !kHalfRows;
   v4u64 scr[2] = {};
   v4i row_scale_rsrc = v4i{0, 0, 0, 0};
   uint64_t tensor_scale_twice = 0;  // zero with row scales
-  if constexpr (kRowScalars) {
+  if constexpr (kRowScalars || kHalfRows) {
     row_scale_rsrc = raw_rsrc(scale_ptr, scale_ld ? (uint32_t)KC * 4u : 4u);
     const uint32_t bits = scale_ld ? 0u : (uint32_t)__builtin_amdgcn_readfirstlane(*static_cast<const int*>(scale_ptr));
     tensor_scale_twice = ((uint64_t)bits << 32) | bits;
@@ -362,7 +374,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   // past the end stay out of range and the walk from slab to slab is scalar arithmetic.
   int q_voff[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) q_voff[i] = NAT ? opaque(nat_live ? (8 * wave + i) * NO + 4 * col4 : kOob) : 0;
+  for (int i = 0; i < 8; ++i) q_voff[i] = NAT && i < NROWS ? opaque(nat_live ? (8 * wave + 4 * row_half + i) * NO + 4 * col4 : kOob) : 0;
   const int q_slab_bytes = 32 * NO;
   const uint64_t q_first = (uint64_t)reinterpret_cast<uintptr_t>(Q) + (uint64_t)q_skip;
   int q_walk_lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)q_first);
@@ -389,6 +401,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   // to outputs that are never stored, the scale only has to come from valid memory.
   auto scale_offset = [&](int s) __attribute__((always_inline)) {
     if constexpr (NS == 0) return 0;
+    else if constexpr (kHalfRows) return opaque(min(s * 32 + 8 * wave + 4 * row_half, KC - 4) * 4);  // four row scales
     else {
       const int n = min(s * 32 + 8 * wave, KC - 8);
       const int k = min(n0 + 4 * col4, NO - 1);  // this thread's first output column (a column of q)
@@ -397,7 +410,11 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
     }
   };
   auto load_scale_piece = [&](int set, int s_off, int i) __attribute__((always_inline)) {
-    if constexpr (SK == KM_WSCALE_E8M0) sraw[set][i] = loop_load_u8(scale_rsrc, s_off + i * scale_ld);
+    if constexpr (kHalfRows) {
+      // range-checked: with one scale for the whole tensor every dword but the one at offset 0 reads as zero
+      const v4i v = loop_load_b128(row_scale_rsrc, s_off);
+      sraw[set][0] = (uint32_t)v[0]; sraw[set][1] = (uint32_t)v[1]; sraw[set][2] = (uint32_t)v[2]; sraw[set][3] = (uint32_t)v[3];
+    } else if constexpr (SK == KM_WSCALE_E8M0) sraw[set][i] = loop_load_u8(scale_rsrc, s_off + i * scale_ld);
     else sraw[set][0] = loop_load_b32(scale_rsrc, s_off);
   };
   // scales that do not go through the counted vector loads: per contraction column of a transposed
@@ -428,6 +445,9 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
                    : "scc");
 #pragma unroll
       for (int i = 0; i < 8; ++i) sc[set][i] = bits_f32((uint32_t)(r[i >> 1] >> (32 * (i & 1))));
+    } else if constexpr (kHalfRows) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sc[set][i] = bits_f32(sraw[set][i] | (uint32_t)tensor_scale_twice);
     }
   };
   auto load_slab = [&](int set, int s) __attribute__((always_inline)) {
@@ -449,7 +469,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   // byte pairs (k, rows 2d and 2d+1) `t1`. Then dword d of unit c (two values of the activation
   // type) comes from one byte pair, and unit c (four dwords) is one 16-byte LDS write.
   uint32_t t1[8], w16[UNITS][4];
-  auto transpose_piece = [&](int set, int p) __attribute__((always_inline)) {  // p < 8
+  auto transpose_piece = [&](int set, int p) __attribute__((always_inline)) {  // p < NROWS
     if constexpr (NAT && QF != KM_Q_INT8) t1[p] = pair_rows(raw[set], p);  // an int8 conversion selects its byte by itself
   };
   auto widen_piece = [&](int set, int c, int d) __attribute__((always_inline)) {
@@ -471,18 +491,22 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   };
   auto store_unit = [&](int stage, int c) __attribute__((always_inline)) {
     uint8_t* slab = b_ring + stage * B_STAGE;
-    const uint4 v = make_uint4(w16[c][0], w16[c][1], w16[c][2], w16[c][3]);
-    if constexpr (!NAT) *reinterpret_cast<uint4*>(slab + slab32_offset(q_row + c * 64, q_chunk)) = v;
-    else if (nat_live) *reinterpret_cast<uint4*>(slab + slab32_offset(nat_row0 + c * nat_stride, wave)) = v;
+    if constexpr (kHalfRows) {
+      *reinterpret_cast<uint2*>(slab + slab32_offset(nat_row0 + c * nat_stride, wave) + 8 * row_half) = make_uint2(w16[c][0], w16[c][1]);
+    } else {
+      const uint4 v = make_uint4(w16[c][0], w16[c][1], w16[c][2], w16[c][3]);
+      if constexpr (!NAT) *reinterpret_cast<uint4*>(slab + slab32_offset(q_row + c * 64, q_chunk)) = v;
+      else if (nat_live) *reinterpret_cast<uint4*>(slab + slab32_offset(nat_row0 + c * nat_stride, wave)) = v;
+    }
   };
   auto commit_all = [&](int set, int stage) __attribute__((always_inline)) {
     merge_scales(set);
 #pragma unroll
-    for (int p = 0; p < 8; ++p) transpose_piece(set, p);
+    for (int p = 0; p < NROWS; ++p) transpose_piece(set, p);
 #pragma unroll
     for (int c = 0; c < UNITS; ++c) {
 #pragma unroll
-      for (int d = 0; d < 4; ++d) widen_piece(set, c, d);
+      for (int d = 0; d < (NAT ? DPC : 4); ++d) widen_piece(set, c, d);
       store_unit(stage, c);
     }
   };
@@ -534,14 +558,15 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
         constexpr int i = decltype(i_tag)::value;
         if constexpr (q == at(i, A_LD, 0, S / 2)) dma_a_pass((u + 3) & 3, a_off, i);
       });
-      static_for<8>([&](auto p_tag) __attribute__((always_inline)) {
+      static_for<NROWS>([&](auto p_tag) __attribute__((always_inline)) {
         constexpr int pp = decltype(p_tag)::value;
-        if constexpr (NAT && q == at(pp, 8, S / 4, S / 2)) transpose_piece(par, pp);
+        if constexpr (NAT && q == at(pp, NROWS, S / 4, S / 2)) transpose_piece(par, pp);
       });
-      static_for<4 * UNITS>([&](auto p_tag) __attribute__((always_inline)) {
+      constexpr int WD = NAT ? DPC : 4;  // widening pieces (dwords) per unit
+      static_for<WD * UNITS>([&](auto p_tag) __attribute__((always_inline)) {
         constexpr int pp = decltype(p_tag)::value;
-        if constexpr (q == at(pp, 4 * UNITS, S / 2, 3 * S / 4)) widen_piece(par, pp / 4, pp % 4);
-        if constexpr (pp % 4 == 3 && q == (at(pp, 4 * UNITS, S / 2, 3 * S / 4) + 1 < S ? at(pp, 4 * UNITS, S / 2, 3 * S / 4) + 1 : S - 1)) store_unit((u + 2) & 3, pp / 4);
+        if constexpr (q == at(pp, WD * UNITS, S / 2, 3 * S / 4)) widen_piece(par, pp / WD, pp % WD);
+        if constexpr (pp % WD == WD - 1 && q == (at(pp, WD * UNITS, S / 2, 3 * S / 4) + 1 < S ? at(pp, WD * UNITS, S / 2, 3 * S / 4) + 1 : S - 1)) store_unit((u + 2) & 3, pp / WD);
       });
       static_for<NL>([&](auto l_tag) __attribute__((always_inline)) {
         constexpr int l = decltype(l_tag)::value;
@@ -614,9 +639,9 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
 #pragma unroll
   for (int b = 0; b < 2; ++b) {
 #pragma unroll
-    for (int i = 0; i < (NAT ? 8 : 2 * UNITS); ++i) asm volatile("" ::"v"(raw[b][i]));
+    for (int i = 0; i < (NAT ? NROWS : 2 * UNITS); ++i) asm volatile("" ::"v"(raw[b][i]));
 #pragma unroll
-    for (int i = 0; i < (NS ? NS : 1); ++i) asm volatile("" ::"v"(sraw[b][i]));
+    for (int i = 0; i < (kHalfRows ? 4 : NS ? NS : 1); ++i) asm volatile("" ::"v"(sraw[b][i]));
     if constexpr (kRowScalars) asm volatile("" ::"s"(scr[b]));
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -673,16 +698,21 @@ inline int launch_config(int config, const void* a, const void* q, const void* s
       return launch_wo<256, 192, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st);
     case 6: {
       // 256 x 256 tiles over as many tile columns as fill whole rounds of the card (one tile per
-      // compute unit and round), 128 x 256 tiles over the rest: the last, partly empty round of large
+      // compute unit and round), half-size tiles over the rest: the last, partly empty round of large
       // tiles becomes a full round of tiles that take less time (8192 x 3072 outputs: 384 large tiles
-      // are one round and a half, so two; 256 large and 256 half tiles are one round each). Every
+      // are one round and a half, so two; 256 large and 256 half tiles are one round each). The half
+      // tile is the one whose step costs least in the mode: 256 x 128 where the codes are read as
+      // stored with a scale per row (its lanes split the rows of a slab), 128 x 256 otherwise. Every
       // output element is the same sum in the same order as in the other configurations.
       const int tm = (M + 255) / 256, tn = (NO + 255) / 256, cus = compute_units();
       if (cus <= 0) return km_fail(KM_ERR_LAUNCH, "km_wo_gemm: cannot ask for the number of compute units");
       const int whole_cols = whole_round_columns(tm, tn, cus);
       int rc = launch_wo<256, 256, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st, 0, whole_cols);
-      if (rc == KM_OK) rc = launch_wo<128, 256, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st, whole_cols, tn - whole_cols);
-      return rc;
+      if (rc != KM_OK) return rc;
+      if constexpr (MODE == kWoDgradN && SK == KM_WSCALE_ROWS)
+        return launch_wo<256, 128, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st, 2 * whole_cols, -1);
+      else
+        return launch_wo<128, 256, DT, QF, MODE, SK>(a, q, scale, scale_ld, bias, c, M, NO, KC, st, whole_cols, -1);
     }
   }
   return km_fail(KM_ERR_ARG, "km_wo_gemm: unknown config");

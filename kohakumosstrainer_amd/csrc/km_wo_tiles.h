@@ -9,7 +9,7 @@
 
 namespace km {
 
-constexpr int kNumWoConfigs = 7;  // 256x256, 128x256, 256x128, 128x128, 64x128, 256x192 (rows x columns of a workgroup's tile); 256x256 with a last round of 128x256
+constexpr int kNumWoConfigs = 7;  // 256x256, 128x256, 256x128, 128x128, 64x128, 256x192 (rows x columns of a workgroup's tile); 256x256 with a last round of half-size tiles
 
 // y = (x @ q^T) * scale + bias over K-contiguous codes q [NO, KC]
 template <int DT>

@@ -105,13 +105,14 @@ def test_input_gradient_of_an_fp8_base_without_a_transposed_copy(recipe, dtype, 
 
 @pytest.mark.parametrize("fmt", ("int8", "fp8"))
 def test_two_tile_shapes_in_one_call(fmt):
-    """The configuration with `tail_bm` covers whole rounds of the card with 256 x 256 tiles and the
-    remaining tile columns with 128 x 256 tiles in a second launch. 17 x 17 large tiles are more
+    """The configuration with `tail` covers whole rounds of the card with 256 x 256 tiles and the
+    remaining tile columns with half-size tiles (128 x 256 forward, 256 x 128 for the gradient) in a
+    second launch. 17 x 17 large tiles are more
     than the card's compute units and not a multiple of them, rows and columns are ragged, and the
     columns of the second launch start in the middle of the output: every element must equal the
     one-shape configuration's bit for bit, forward (bias and scale follow the column window) and
     input gradient."""
-    mixed = [c["id"] for c in native.configs(native.KERNEL_WO_FWD) if c.get("tail_bm", 0)]
+    mixed = [c["id"] for c in native.configs(native.KERNEL_WO_FWD) if c.get("tail", 0)]
     assert mixed, "no configuration with a tail"
     m, wide, deep = 4100, 4200, 264
     x, q, scale, bias, _ = case(m, wide, deep, fmt, torch.bfloat16, seed=3)  # forward: 4200 output columns
@@ -130,7 +131,7 @@ def test_two_tile_shapes_under_graph_capture():
     """Both launches of the two-shape configuration, and its question to the runtime about the
     number of compute units, inside a captured stream: every replay equals the eager result (inputs
     refilled between replays, eager work in between)."""
-    mixed = [c["id"] for c in native.configs(native.KERNEL_WO_FWD) if c.get("tail_bm", 0)][0]
+    mixed = [c["id"] for c in native.configs(native.KERNEL_WO_FWD) if c.get("tail", 0)][0]
     m, n, k = 4100, 264, 4200
     _, q, scale, _, dy = case(m, n, k, "fp8", torch.bfloat16, seed=6)
     dq, dscale, static_dy = q.cuda(), scale.cuda(), dy.cuda()
