@@ -666,7 +666,7 @@ template <int BM, int BN, int DT, int QF, int MODE, int SK>
 inline int launch_wo(const void* a, const void* q, const void* scale, int scale_ld, const void* bias, void* c, int M, int NO,
                      int KC, hipStream_t st, int tn_first = 0, int tn_count = -1) {
   if (tn_count < 0) tn_count = (NO + BN - 1) / BN - tn_first;  // to the last tile column
-  if (tn_count == 0) return KM_OK;
+  if (tn_count <= 0) return KM_OK;  // nothing left (a window that starts past the last, narrower tile column)
   const int tiles = ((M + BM - 1) / BM) * tn_count;
   hipLaunchKernelGGL((wo_gemm_kernel<BM, BN, DT, QF, MODE, SK>), dim3(tiles), dim3(256), 0, st, (const uint16_t*)a,
                      (const uint8_t*)q, scale, scale_ld, (const uint16_t*)bias, (uint16_t*)c, M, NO, KC, tn_first, tn_count);

@@ -127,6 +127,20 @@ def test_two_tile_shapes_in_one_call(fmt):
         assert torch.equal(native.wo_gemm_dgrad(dy.cuda(), q2.cuda(), scale2.cuda(), cfg), dx0)
 
 
+def test_two_tile_shapes_when_the_large_tiles_cover_everything():
+    """256 x 2 large tiles are whole rounds of a card with 256 (or 128, 64 ...) compute units, and the
+    last tile column is only 128 wide: the window of the half-size tiles starts past the last
+    128-column tile and must come out empty, not negative."""
+    mixed = [c["id"] for c in native.configs(native.KERNEL_WO_FWD) if c.get("tail", 0)][0]
+    m, n, k = 65536, 64, 384
+    _, q, scale, _, dy = case(m, n, k, "fp8", torch.bfloat16, seed=8)
+    dx0 = native.wo_gemm_dgrad(dy.cuda(), q.cuda(), scale.cuda(), 0)
+    assert torch.equal(native.wo_gemm_dgrad(dy.cuda(), q.cuda(), scale.cuda(), mixed), dx0)
+    x, q, scale, bias, _ = case(m, k, n, "fp8", torch.bfloat16, seed=9)
+    y0 = native.wo_gemm_fwd(x.cuda(), q.cuda(), scale.cuda(), bias.cuda(), 0)
+    assert torch.equal(native.wo_gemm_fwd(x.cuda(), q.cuda(), scale.cuda(), bias.cuda(), mixed), y0)
+
+
 def test_two_tile_shapes_under_graph_capture():
     """Both launches of the two-shape configuration, and its question to the runtime about the
     number of compute units, inside a captured stream: every replay equals the eager result (inputs
