@@ -79,6 +79,25 @@ def test_weight_only_gemms_with_codes_just_below_one_gib():
     assert torch.equal(back, (q[rows].float() * scale[rows, None]).to(torch.bfloat16))
 
 
+@pytest.mark.gpu
+def test_input_gradient_over_few_very_long_rows_of_codes():
+    """Eight rows of 2^26 + 256 codes: 32 rows of such a q would pass 2^31 bytes, the stride by
+    which the tiled kernels step through q, so the entry point must take another path. One-hot
+    gradient rows read the rounded weight back, every element of every row."""
+    n, k = 8, 2**26 + 256
+    assert n * k <= 2**30 - 1 and 32 * k > 2**31 - 1
+    dev = torch.device("cuda")
+    g = torch.Generator(device=dev).manual_seed(4)
+    q = torch.randint(-127, 128, (n, k), generator=g, device=dev, dtype=torch.int8)
+    scale = torch.rand(n, generator=g, device=dev) * 1e-3 + 1e-4
+    probe = torch.eye(n, device=dev, dtype=torch.bfloat16)
+    for cfg in (0, 2):
+        back = native.wo_gemm_dgrad(probe, q, scale, cfg)
+        for r in range(n):
+            assert torch.equal(back[r], (q[r].float() * scale[r]).to(torch.bfloat16)), f"cfg{cfg} row {r}"
+        del back
+
+
 def _rc(fn, *args):
     rc = fn(*args)
     return rc, native.load().km_last_error().decode()
