@@ -9,6 +9,7 @@ made per call as the reference makes its column-major copy (`int8/formats.py:55-
 
 from kohakumosstrainer_amd import native
 from kohakumosstrainer_amd.kernels import registry, tuning
+from kohakumosstrainer_amd.kernels.backends.hip import quant as wo
 from kohakumosstrainer_amd.kernels.constraints import requires
 from kohakumosstrainer_amd.kernels.hadamard import HALF
 from kohakumosstrainer_amd.kernels.hadamard import rotate_2d
@@ -57,7 +58,7 @@ def dgrad(dy, q, scale, group, mode):
     m, n = dy.shape
     k = q.shape[1]
     if mode == "16bit":
-        dx = native.wo_gemm_dgrad(dy, q.contiguous(), scale, 0)
+        dx = wo.dgrad(dy, q.contiguous(), scale)  # the weight-only kernel over the stored codes, its tuned tile
         return rotate_2d(dx, group) if group else dx
     _check("dgrad", n)
     gq, gs = native.quant_rows_i8(dy, scale)
