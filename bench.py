@@ -152,7 +152,18 @@ def other_configs(dev, reps):
         best[name] = min(times.items(), key=lambda kv: kv[1])
     flop = 2 * m * n * k
     (fc, f), (dc, d) = best["fwd"], best["dgrad"]
-    out["mx_frozen_base_M2048_K4096_N12288"] = {"fwd_ms": f, "fwd_TFLOPs": flop / f / 1e9, "fwd_config": fc, "dgrad_ms": d, "dgrad_TFLOPs": flop / d / 1e9, "dgrad_config": dc, "peak_TFLOPs": FP8_PEAK_TFLOPS, "note": "quantizer + GEMM per call"}
+    # the 16-bit input gradient of the same base (no transposed fp8 copy kept): dy in bf16 against the
+    # codes as stored, widened in registers with their E8M0 scales; bf16 MFMA, so priced at the bf16 peak
+    codes, nat = native.quant_mx(w)[:2]
+    codes = codes.view(torch.float8_e4m3fn)
+    w16 = {}
+    for cfg in (0, 2, 3):  # the tiles built for E8M0-scaled bases: 256 x 256, 256 x 128, 128 x 128
+        native.wo_gemm_dgrad(dy, codes, nat, cfg, "mx")
+        w16[cfg] = event_ms(lambda: native.wo_gemm_dgrad(dy, codes, nat, cfg, "mx"), reps)
+    wc, wt = min(w16.items(), key=lambda kv: kv[1])
+    out["mx_frozen_base_M2048_K4096_N12288"] = {"fwd_ms": f, "fwd_TFLOPs": flop / f / 1e9, "fwd_config": fc, "dgrad_ms": d, "dgrad_TFLOPs": flop / d / 1e9, "dgrad_config": dc, "peak_TFLOPs": FP8_PEAK_TFLOPS, "note": "quantizer + GEMM per call",
+                                                 "dgrad_w16_ms": wt, "dgrad_w16_TFLOPs": flop / wt / 1e9, "dgrad_w16_config": wc, "dgrad_w16_peak_TFLOPs": 2500.0}
+    del codes, nat
     # the row recipe (one fp32 scale per activation row and per weight row) at the headline shape
     m, k, n = 16384, 3072, 9216
     x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(dev)

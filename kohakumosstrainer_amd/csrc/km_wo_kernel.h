@@ -266,11 +266,12 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   // Codes as stored, 128 columns, a scale per row: the 32 dwords of a row n keep half a wavefront
   // busy, so the halves take four rows n each (everything per lane and step halves: loads,
   // permutes, conversions; a lane writes 8 bytes per column instead of 16).
-  constexpr bool kHalfRows = NAT && BN == 128 && SK == KM_WSCALE_ROWS;
+  constexpr bool kHalfRows = NAT && BN == 128 && (SK == KM_WSCALE_ROWS || SK == KM_WSCALE_E8M0);
+  constexpr bool kHalfRowScales = kHalfRows && SK == KM_WSCALE_ROWS;  // four fp32 row scales in one vector load
   constexpr int NROWS = kHalfRows ? 4 : 8;             // rows n per lane (codes as stored)
   constexpr int DPC = NROWS / 2;                       // dwords of two values per column
   constexpr int NQ = NAT ? NROWS : UNITS;              // code loads per thread and step
-  constexpr int NS = !NAT ? 0 : SK == KM_WSCALE_E8M0 ? 8 : (SK == KM_WSCALE_BLOCKS || kHalfRows) ? 1 : 0;  // scale loads through the vector path
+  constexpr int NS = !NAT ? 0 : SK == KM_WSCALE_E8M0 ? NROWS : (SK == KM_WSCALE_BLOCKS || kHalfRowScales) ? 1 : 0;  // scale loads through the vector path
   constexpr int NV = A_LD + NQ + NS;                   // vector-memory loads issued per step, counted by hand below
   static_assert(!NAT || BN == 256 || BN == 192 || BN == 128, "the transposing load covers 256, 192 or 128 columns");
   static_assert(NV < 48, "vmcnt holds 6 bits");
@@ -335,7 +336,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   v4u64 scr[2] = {};
   v4i row_scale_rsrc = v4i{0, 0, 0, 0};
   uint64_t tensor_scale_twice = 0;  // zero with row scales
-  if constexpr (kRowScalars || kHalfRows) {
+  if constexpr (kRowScalars || kHalfRowScales) {
     row_scale_rsrc = raw_rsrc(scale_ptr, scale_ld ? (uint32_t)KC * 4u : 4u);
     const uint32_t bits = scale_ld ? 0u : (uint32_t)__builtin_amdgcn_readfirstlane(*static_cast<const int*>(scale_ptr));
     tensor_scale_twice = ((uint64_t)bits << 32) | bits;
@@ -401,16 +402,16 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   // to outputs that are never stored, the scale only has to come from valid memory.
   auto scale_offset = [&](int s) __attribute__((always_inline)) {
     if constexpr (NS == 0) return 0;
-    else if constexpr (kHalfRows) return opaque(min(s * 32 + 8 * wave + 4 * row_half, KC - 4) * 4);  // four row scales
+    else if constexpr (kHalfRowScales) return opaque(min(s * 32 + 8 * wave + 4 * row_half, KC - 4) * 4);  // four row scales
     else {
-      const int n = min(s * 32 + 8 * wave, KC - 8);
+      const int n = min(s * 32 + 8 * wave + 4 * row_half, KC - NROWS);
       const int k = min(n0 + 4 * col4, NO - 1);  // this thread's first output column (a column of q)
       if constexpr (SK == KM_WSCALE_E8M0) return opaque(n * scale_ld + (k >> 5));
       else return opaque(((n >> 7) * scale_ld + (k >> 7)) * 4);  // n .. n + 7 share a block
     }
   };
   auto load_scale_piece = [&](int set, int s_off, int i) __attribute__((always_inline)) {
-    if constexpr (kHalfRows) {
+    if constexpr (kHalfRowScales) {
       // range-checked: with one scale for the whole tensor every dword but the one at offset 0 reads as zero
       const v4i v = loop_load_b128(row_scale_rsrc, s_off);
       sraw[set][0] = (uint32_t)v[0]; sraw[set][1] = (uint32_t)v[1]; sraw[set][2] = (uint32_t)v[2]; sraw[set][3] = (uint32_t)v[3];
@@ -445,7 +446,7 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
                    : "scc");
 #pragma unroll
       for (int i = 0; i < 8; ++i) sc[set][i] = bits_f32((uint32_t)(r[i >> 1] >> (32 * (i & 1))));
-    } else if constexpr (kHalfRows) {
+    } else if constexpr (kHalfRowScales) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) sc[set][i] = bits_f32(sraw[set][i] | (uint32_t)tensor_scale_twice);
     }

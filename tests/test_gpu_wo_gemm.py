@@ -94,10 +94,14 @@ def test_input_gradient_of_an_fp8_base_without_a_transposed_copy(recipe, dtype, 
     dy = torch.randn(m, n, generator=g).to(dtype)
     truth = dy.double() @ w64
     eager = linear.fp8_dgrad(dy, q, scale, None, None, None, recipe)
+    first = None
     for cfg in range(n_configs()):
         dx = native.wo_gemm_dgrad(dy.cuda(), q.cuda(), scale.cuda(), cfg, recipe)
         assert dx.shape == (m, k) and dx.dtype == dtype
         assert_no_regression(dx.cpu(), eager, truth, f"w16 dgrad {recipe} cfg{cfg} {m}x{n}x{k}")
+        # every tile shape (and lane layout) sums a row's products in the same order
+        first = dx if first is None else first
+        assert torch.equal(dx, first), f"{recipe} cfg{cfg} differs from cfg0"
     eye = torch.eye(n, dtype=dtype)[:256]
     back = native.wo_gemm_dgrad(eye.cuda(), q.cuda(), scale.cuda(), 0, recipe).cpu()
     assert torch.equal(back, formats.dequantize(q, scale, recipe, dtype)[:256])
