@@ -263,10 +263,10 @@ __global__ __launch_bounds__(256) void wo_gemm_kernel(const uint16_t* __restrict
   constexpr bool NAT = MODE == kWoDgradN;
   constexpr bool PRESCALE = MODE != kWoFwd;
   constexpr int UNITS = NAT ? 4 : BN / 64;             // 16-byte LDS writes per thread and step
-  // Codes as stored, 128 columns, a scale per row: the 32 dwords of a row n keep half a wavefront
-  // busy, so the halves take four rows n each (everything per lane and step halves: loads,
-  // permutes, conversions; a lane writes 8 bytes per column instead of 16).
-  constexpr bool kHalfRows = NAT && BN == 128 && (SK == KM_WSCALE_ROWS || SK == KM_WSCALE_E8M0);
+  // Codes as stored, 128 columns: the 32 dwords of a row n keep half a wavefront busy, so the
+  // halves take four rows n each (everything per lane and step halves: loads, permutes,
+  // conversions, scale bytes; a lane writes 8 bytes per column instead of 16).
+  constexpr bool kHalfRows = NAT && BN == 128;
   constexpr bool kHalfRowScales = kHalfRows && SK == KM_WSCALE_ROWS;  // four fp32 row scales in one vector load
   constexpr int NROWS = kHalfRows ? 4 : 8;             // rows n per lane (codes as stored)
   constexpr int DPC = NROWS / 2;                       // dwords of two values per column
