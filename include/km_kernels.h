@@ -222,6 +222,18 @@ int km_wo_gemm_dgrad_static(const void *dy, const void *q, const float *scale, v
 int km_group_hadamard(const void *x, int64_t rows, int64_t cols, int dtype, int group, void *y,
                       void *stream);
 
+/* Measurement only, no counterpart in the reference: the block-scaled fp8 MFMA run out of registers
+ * (one wavefront per SIMD on every compute unit, 64 independent 16x16x128 MFMAs per trip over eight
+ * fragments of each operand, no loads, no LDS, no barriers), `trips` trips per wavefront. a_frags and
+ * b_frags are 16 KiB of e4m3 codes each (8 fragments x 64 lanes x 32 bytes, 32-byte aligned): a
+ * benchmark passes rows of its real operands so that the data-dependent power draw matches. sink
+ * takes 256 floats per compute unit. *flop_out receives the launch's flop count; flop / device
+ * time is the rate the card's clocks sustain on its matrix pipes, the ceiling of the GEMMs above
+ * (the method of the reference's docs/performance/gemm-efficiency.md:28-29: peak from the measured
+ * clock, not the nominal one). */
+int km_probe_mfma_ceiling(const void *a_frags, const void *b_frags, void *sink, int64_t sink_floats,
+                          int trips, int64_t *flop_out, void *stream);
+
 /* Tile configurations per kernel, for the host-side tuning table (the reference enumerates its
  * Triton tiles in backends/triton/fp8/linear.py:39-75 and backends/triton/quant.py:132-141).
  * km_config_desc writes "key=value,..." (bm, bn: rows and columns of a work-group's tile; for the

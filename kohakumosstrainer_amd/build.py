@@ -19,7 +19,7 @@ OUT_DIR = PKG / "_lib"
 LIB = OUT_DIR / "libkm_kernels.so"
 HOST_LIB = OUT_DIR / "libkm_hostcheck.so"
 SOURCES = ("km_api.hip", "km_quant.hip", "km_gemm_fp8.hip", "km_gemm_fp8_w32.hip", "km_gemm_blocks.hip", "km_gemm_fused.hip", "km_wo_gemm.hip", "km_wo_dgrad.hip", "km_wo_fwd_bf16.hip", "km_wo_fwd_f16.hip", "km_wo_dgrad_bf16_i8.hip", "km_wo_dgrad_bf16_e4m3.hip", "km_wo_dgrad_bf16_e4m3b.hip",
-           "km_wo_dgrad_f16_i8.hip", "km_wo_dgrad_f16_e4m3.hip", "km_wo_dgrad_f16_e4m3b.hip", "km_hadamard.hip")
+           "km_wo_dgrad_f16_i8.hip", "km_wo_dgrad_f16_e4m3.hip", "km_wo_dgrad_f16_e4m3b.hip", "km_hadamard.hip", "km_probe.hip")
 ARCH = "gfx950"
 # packed fp32 instructions are switched off for every device translation unit
 DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

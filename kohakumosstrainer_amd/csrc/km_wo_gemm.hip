@@ -102,7 +102,10 @@ int wo_config_desc(int config, char* buf, int len) {
 template <int DT, int QF, bool DGRAD>
 static int dispatch_wo(int config, const void* a, const void* q, const float* scale, const void* bias, void* c, int M,
                        int NO, int KC, hipStream_t st) {
-  if (KC % 8 || ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(q)) & 15)) {
+  // The tiles read A through a descriptor based at the tile's first row with 32-bit byte offsets: 256
+  // rows of A must stay below 2^31 bytes. The forward's A is capped as a whole; the gradient dy[M, KC]
+  // is not, so a very long contraction takes the element-wise kernel.
+  if (KC % 8 || (DGRAD && KC > kMaxTiledRowElems) || ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(q)) & 15)) {
     const int64_t n = (int64_t)M * NO;
     hipLaunchKernelGGL((wo_gemm_scalar<DT, QF, DGRAD>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
                        (const uint16_t*)a, (const uint8_t*)q, scale, (const uint16_t*)bias, (uint16_t*)c, M, NO, KC);

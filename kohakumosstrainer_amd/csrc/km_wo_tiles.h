@@ -35,6 +35,9 @@ inline int wo_tiles_dgrad_n(int q_format, int scale_kind, int config, const void
   return wo_tiles_dgrad_n_part<DT, kWoPartE4m3Blocks>(scale_kind, config, dy, q, scale, scale_ld, dx, M, N, K, st);
 }
 
+// longest row of a 16-bit operand that a 256-row tile can address with 32-bit byte offsets
+constexpr int kMaxTiledRowElems = 0x7FFFFFFF / (256 * 2);
+
 // argument checks shared by the entry points
 int check_wo_args(const char* who, const void* a, const void* q, const void* scale, void* c, int64_t M, int64_t N, int64_t K,
                   int q_format, int dtype, int config);

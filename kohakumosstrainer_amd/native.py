@@ -49,6 +49,7 @@ EXPORTS = (
     "km_wo_gemm_dgrad_w16",
     "km_wo_gemm_dgrad_static",
     "km_group_hadamard",
+    "km_probe_mfma_ceiling",
     "km_num_configs",
     "km_config_desc",
 )
@@ -90,6 +91,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.km_wo_gemm_dgrad_w16.argtypes = [p, p, p, i32, i64, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_wo_gemm_dgrad_static.argtypes = [p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_group_hadamard.argtypes = [p, i64, i64, i32, i32, p, p]
+    lib.km_probe_mfma_ceiling.argtypes = [p, p, p, i64, i32, c.POINTER(c.c_int64), p]
     lib.km_num_configs.argtypes = [i32]
     lib.km_config_desc.argtypes = [i32, i32, c.c_char_p, i32]
     for name in EXPORTS:
@@ -304,6 +306,25 @@ def group_hadamard(x: Tensor, group: int) -> Tensor:
     with torch.cuda.device(x.device):
         _check(load().km_group_hadamard(x.data_ptr(), x.shape[0], x.shape[1], _dtype_code(x.dtype), int(group), y.data_ptr(), _stream(x)))
     return y
+
+
+def mfma_ceiling_probe(a_codes: Tensor, b_codes: Tensor, trips: int) -> int:
+    """Launch the registers-only block-scaled fp8 MFMA loop (`km_probe_mfma_ceiling`) on the current
+    stream with the first 16 KiB of `a_codes` / `b_codes` (e4m3 codes of real operands) as its
+    fragments; returns the launch's flop count. A measurement aid: time it with events."""
+    dev = _on_gpu(a_codes, b_codes)
+    frags = []
+    for t in (a_codes, b_codes):
+        flat = t.contiguous().view(torch.uint8).reshape(-1)
+        if flat.numel() < 16384:
+            raise ValueError("the probe takes at least 16 KiB of codes per operand")
+        frags.append(flat[:16384])
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    sink = torch.empty(cus * 256, dtype=torch.float32, device=dev)
+    flop = ctypes.c_int64(0)
+    with torch.cuda.device(dev):
+        _check(load().km_probe_mfma_ceiling(frags[0].data_ptr(), frags[1].data_ptr(), sink.data_ptr(), sink.numel(), int(trips), ctypes.byref(flop), _stream(a_codes)))
+    return flop.value
 
 
 # ---- GEMMs --------------------------------------------------------------------------------

@@ -17,7 +17,7 @@ from collections.abc import Callable
 import torch
 from torch import nn
 
-from kohakumosstrainer_amd.model.linear import MossLinear
+from kohakumosstrainer_amd.model.linear import MossLinear, placeholder
 from kohakumosstrainer_amd.quant.bind import work_device as default_work_device
 from kohakumosstrainer_amd.quant.compute import COMPUTE, ComputeCache, ComputeWeight, eligible, recipe_of
 from kohakumosstrainer_amd.quant.weights import FORMATS, QuantWeight
@@ -39,11 +39,12 @@ def accepts(fmt: str, out_features: int, in_features: int) -> bool:
 
 
 def default_filter(keep_fp32: tuple[str, ...], min_features: int = 256) -> Callable[[str, nn.Linear], bool]:
-    """Accept a linear unless its name contains one of `keep_fp32` or it is narrower than
-    `min_features` on either side."""
+    """Accept a linear unless it is one of `keep_fp32` or lies under one (`name == key` or
+    `name` starts with `key.`; a name that merely contains a key is not kept), or it is narrower
+    than `min_features` on either side."""
 
     def accept(name: str, lin: nn.Linear) -> bool:
-        if any(part in name for part in keep_fp32):
+        if any(name == key or name.startswith(key + ".") for key in keep_fp32):
             return False
         return min(lin.in_features, lin.out_features) >= min_features
 
@@ -51,7 +52,8 @@ def default_filter(keep_fp32: tuple[str, ...], min_features: int = 256) -> Calla
 
 
 class QuantLinear(nn.Module):
-    """A plain `nn.Linear` replaced by a quantized base and its (dense) bias."""
+    """A plain `nn.Linear` replaced by a quantized base and its (dense) bias. The base is the
+    submodule `qweight`: state keys are `qweight.q`, `qweight.scale`, ... and `bias`."""
 
     def __init__(self, linear: nn.Linear, fmt: str, compute_dtype: torch.dtype, recipe: str = "row", work_device=None):
         super().__init__()
@@ -61,7 +63,8 @@ class QuantLinear(nn.Module):
 
     def _adopt(self, in_features, out_features, base, bias, compute_dtype) -> None:
         self.in_features, self.out_features, self.compute_dtype = in_features, out_features, compute_dtype
-        self.base = base
+        self.qweight = base
+        base.bind(compute_dtype)
         self.bias = None if bias is None else nn.Parameter(bias.detach().clone(), requires_grad=False)
 
     @classmethod
@@ -73,7 +76,7 @@ class QuantLinear(nn.Module):
 
     def forward(self, x):
         bias = None if self.bias is None else self.bias.to(x.dtype)
-        return self.base.linear(x, bias)
+        return self.qweight.linear(x, bias)
 
 
 def _walk_children(module: nn.Module, prefix: str = ""):
@@ -139,6 +142,7 @@ def quantize_model(model: nn.Module, fmt: str, accept=None, compute_dtype: torch
         dense_bytes += layer.weight.numel() * layer.weight.element_size()
         base = make_base(layer.weight.detach().to(where), fmt, recipe, dgrad).to(home)
         quant_bytes += base.nbytes()
+        layer.weight = placeholder(layer.weight)
         layer.set_base(base)
         if compute_dtype is not None:
             base.bind(compute_dtype, home)

@@ -98,6 +98,31 @@ def test_input_gradient_over_few_very_long_rows_of_codes():
         del back
 
 
+@pytest.mark.gpu
+def test_input_gradient_with_a_contraction_too_long_for_tile_offsets():
+    """dy[M, N] with N = 2^22: 256 rows of it are 2^31 bytes, one more than a tile's 32-bit offsets
+    reach, so the entry point must not hand this shape to the tiled kernels. One-hot gradient rows
+    (the last rows of what would be a 256-row tile and the rows after it included) read single
+    rows of the rounded weight back exactly."""
+    n, k, m = 2**22, 8, 260
+    assert n > (2**31 - 1) // 512
+    dev = torch.device("cuda")
+    g = torch.Generator(device=dev).manual_seed(5)
+    q = torch.randint(-127, 128, (n, k), generator=g, device=dev, dtype=torch.int8)
+    scale = torch.rand(n, generator=g, device=dev) * 1e-3 + 1e-4
+    dy = torch.zeros(m, n, device=dev, dtype=torch.bfloat16)
+    picks = {0: 0, 1: n - 1, 127: n // 2 + 3, 254: 17, 255: n - 1, 256: n - 9, 259: n - 2}
+    for r, c in picks.items():
+        dy[r, c] = 1.0
+    dx = native.wo_gemm_dgrad(dy, q, scale, 0)
+    want = torch.zeros(m, k, device=dev, dtype=torch.bfloat16)
+    for r, c in picks.items():
+        want[r] = (q[c].float() * scale[c]).to(torch.bfloat16)
+    assert torch.equal(dx, want)
+    ws = native.wo_gemm_dgrad_workspace(dy, q, scale, 0)
+    assert torch.equal(ws, want)
+
+
 def _rc(fn, *args):
     rc = fn(*args)
     return rc, native.load().km_last_error().decode()

@@ -162,3 +162,94 @@ def test_compute_cache_train_op_gives_weight_gradient():
     assert torch.equal(lin.compute.q.view(torch.uint8), old.view(torch.uint8)) and not torch.equal(lin.compute.scale, formats.quantize(lin.weight / 4, "mx")[1])
     lin.set_compute(None)
     assert lin.is_plain
+
+
+def test_fp32_layer_takes_16bit_activations():
+    """A layer kept in fp32 (a conditioning projection) runs in the activation's type: weight and
+    bias are cast per call (reference `src/kohakumoss/model/linear.py:79-83`)."""
+    for bias in (True, False):
+        lin = MossLinear(64, 48, bias=bias)
+        lin.init_weights(0.05)
+        if bias:
+            nn.init.normal_(lin.bias, std=0.1)
+        x = torch.randn(5, 64).to(torch.bfloat16)
+        y = lin(x)
+        assert y.dtype == torch.bfloat16
+        want = nn.functional.linear(x, lin.weight.to(torch.bfloat16), lin.bias.to(torch.bfloat16) if bias else None)
+        assert torch.equal(y, want)
+        assert lin.weight.dtype == torch.float32
+
+
+def test_set_base_none_keeps_the_dense_weight():
+    lin = MossLinear(256, 256, bias=False)
+    lin.init_weights(0.05)
+    dense = lin.weight.detach().clone()
+    x = torch.randn(3, 256)
+    ref = lin(x)
+    lin.set_base(None)
+    assert lin.base is None and lin.is_plain and torch.equal(lin.weight, dense)
+    assert torch.equal(lin(x), ref)
+    # attaching does not touch the parameter either: whoever attaches decides about it
+    base = QuantWeight.from_weight(dense, "int8")
+    lin.set_base(base)
+    assert lin.base is base and not lin.is_plain and torch.equal(lin.weight, dense)
+    close(lin(x), ref, 1e-2)
+    lin.set_base(None)
+    assert lin.base is None and "base" not in lin._modules and torch.equal(lin(x), ref)
+    # a base that is no module (a streamed handle) attaches and detaches the same way
+    class Handle:
+        def linear(self, x, bias):
+            return x[:, :1] * 0 + 7.0
+    lin.set_base(Handle())
+    assert float(lin(x)[0, 0]) == 7.0
+    lin.clear_base()
+    assert torch.equal(lin(x), ref)
+
+
+def test_is_plain_sees_a_patched_forward_and_init_is_gaussian():
+    lin = MossLinear(64, 64)
+    assert lin.is_plain
+    lin.forward = lambda x: x  # what an adapter library does to the instance
+    assert not lin.is_plain
+    del lin.forward
+    assert lin.is_plain
+    big = MossLinear(512, 512, bias=True)
+    torch.manual_seed(3)
+    big.init_weights(0.02)
+    torch.manual_seed(3)
+    want = torch.empty(512, 512).normal_(std=0.02)
+    assert torch.equal(big.weight.detach(), want), "init_weights draws the weight with normal_ (same stream)"
+    assert float(big.weight.detach().abs().max()) > 3 * 0.02, "an untruncated normal has tails beyond 3 sigma at this size"
+    assert torch.count_nonzero(big.bias) == 0
+
+
+def test_deleted_weight_leaves_a_typed_stand_in():
+    lin = MossLinear(32, 16, dtype=torch.bfloat16)
+    assert lin.weight_like is lin.weight
+    del lin.weight
+    held = lin.weight_like
+    assert held.numel() == 0 and held.dtype == torch.bfloat16
+    lin.to(torch.float16)
+    assert lin.weight_like.dtype == torch.float16
+
+
+def test_keep_filter_is_by_prefix_not_substring():
+    accept = default_filter(("t_embedder", "final"), min_features=16)
+    lin = MossLinear(64, 64)
+    assert not accept("t_embedder", lin) and not accept("t_embedder.mlp.0", lin) and not accept("final.proj", lin)
+    assert accept("blocks.0.t_embedder_proj", lin), "a name that only contains a kept key is quantized"
+    assert accept("blocks.3.final", lin) and accept("t_embedder2.x", lin)
+    assert not accept("x", MossLinear(8, 64))
+
+
+def test_quantlinear_state_keys_use_qweight():
+    """State of a QuantLinear must load on the other side: the base sits under `qweight`
+    (reference `src/kohakumoss/quant/convert.py:78-79`)."""
+    plain = nn.Linear(256, 256)
+    ql = QuantLinear(plain, "int8", torch.float32)
+    keys = set(ql.state_dict())
+    assert {"qweight.q", "qweight.scale", "bias"} <= keys and not any(k.startswith("base.") for k in keys), keys
+    other = QuantLinear(nn.Linear(256, 256), "int8", torch.float32)
+    other.load_state_dict(ql.state_dict())
+    x = torch.randn(2, 256)
+    assert torch.equal(other(x), ql(x))
