@@ -135,6 +135,29 @@ def cpu_other_configs(x_host):
     return out
 
 
+def mfma_ceiling(a_codes, b_codes):
+    """What the card's clocks sustain on the matrix pipes: the block-scaled fp8 MFMA out of registers
+    (one wavefront per SIMD on every compute unit, the GEMM's 64 accumulator tiles and 8 + 8 operand
+    fragments taken from the benchmark's own codes, no loads, no LDS, no barriers), about 60 ms per
+    launch after a launch of the same length to settle the clocks. The implied clock assumes the
+    pipe's nominal 8192 flop per cycle and compute unit (dense fp8)."""
+    from kohakumosstrainer_amd import native
+
+    trips = 50_000  # 64 MFMAs of 32 cycles each per trip: about 1.1 us
+    native.mfma_ceiling_probe(a_codes, b_codes, trips)
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    flop = native.mfma_ceiling_probe(a_codes, b_codes, trips)
+    end.record()
+    end.synchronize()
+    ms = start.elapsed_time(end)
+    tflops = flop / ms / 1e9
+    cus = torch.cuda.get_device_properties(a_codes.device).multi_processor_count
+    return {"TFLOPs": tflops, "ms": ms, "frac_of_nominal": tflops / FP8_PEAK_TFLOPS, "implied_clock_GHz": tflops * 1e12 / (cus * 8192) / 1e9,
+            "compute_units": cus, "kernel": "mfma_ceiling_kernel: v_mfma_scale_f32_16x16x128_f8f6f4 from registers only, 4 wavefronts per compute unit"}
+
+
 def other_configs(dev, reps):
     """Device time of the other kernels of the path at their benchmark shapes (event-timed,
     back to back): weight-only int8 / e4m3 GEMMs, the frozen-base MXFP8 forward + input
@@ -240,6 +263,30 @@ def other_configs(dev, reps):
         "quant_rows_us": qt * 1e3, "quant_rows_GBps": (m * k * 3 + m * 4) / qt / 1e6, "hbm_peak_GBps": HBM_PEAK_GBS,
         "gemm_ms": gt, "gemm_TFLOPs": flop / gt / 1e9, "step_ms": st, "step_TFLOPs": flop / st / 1e9, "peak_TFLOPs": FP8_PEAK_TFLOPS,
     }
+    # the per-tensor recipe (one fp32 scale for x, one for W), same shape: abs-max pass + cast, fp8 MFMA GEMM
+    wtq, wts = native.quant_tensor(w)
+    xtq, xts = native.quant_tensor(x)
+    sbuf1 = torch.empty(1, dtype=torch.float32, device=dev)
+    amax_work = torch.empty(1, dtype=torch.int32, device=dev)
+
+    def quant_tensor_only():  # the bare entry point: no output allocation in the timed region
+        lib.km_quant_tensor(x.data_ptr(), m, k, k, 1, native.KM_BF16, qbuf.data_ptr(), sbuf1.data_ptr(), amax_work.data_ptr(), stream)
+
+    quant_tensor_only()
+    qt = event_ms(quant_tensor_only, reps)
+    gt = event_ms(lambda: native.gemm_fp8_tensor(xtq, xts, wtq, wts.reshape(1), bias, torch.bfloat16, 0), reps)
+
+    def tensor_step():
+        aq, sa = native.quant_tensor(x)
+        return native.gemm_fp8_tensor(aq, sa, wtq, wts.reshape(1), bias, torch.bfloat16, 0)
+
+    tensor_step()
+    st = event_ms(tensor_step, reps)
+    out["tensor_recipe_M16384_K3072_N9216"] = {
+        "quant_tensor_us": qt * 1e3, "quant_tensor_GBps": (m * k * 5) / qt / 1e6, "hbm_peak_GBps": HBM_PEAK_GBS,
+        "quant_note": "two passes (abs-max over x, then the cast): 2 + 2 bytes read and 1 written per element, the second read mostly from the last-level cache",
+        "gemm_ms": gt, "gemm_TFLOPs": flop / gt / 1e9, "step_ms": st, "step_TFLOPs": flop / st / 1e9, "peak_TFLOPs": FP8_PEAK_TFLOPS,
+    }
     # the block recipe (fp32 scales per row x 128 columns / per 128 x 128 weight block), same shape
     wbq, wbs = native.quant_blocks(w, "weight")
     xbq, _, xbs = native.quant_blocks(x, "act", natural=False, kmajor=True)  # the GEMM reads the [K/128, M] scale copy
@@ -331,9 +378,27 @@ def other_configs(dev, reps):
     qt = event_ms(quant8_only, reps)
     gt = event_ms(lambda: native.gemm_i8_rows(x8, x8s, w8, w_scale, bias, torch.bfloat16, 0), reps)
     st = event_ms(int8_step, reps)
+    # a rotated base (ConvRot, groups of 256): the quantizer rotates the rows on their way in; against
+    # the rotation kernel followed by the quantizer
+    def quant8_rotated():
+        lib.km_quant_rows_i8_rotated(x.data_ptr(), m, k, k, native.KM_BF16, 256, q8buf.data_ptr(), sbuf.data_ptr(), stream)
+
+    xrot = torch.empty_like(x)
+
+    def rotate_then_quant8():
+        lib.km_group_hadamard(x.data_ptr(), m, k, native.KM_BF16, 256, xrot.data_ptr(), stream)
+        lib.km_quant_rows_i8(xrot.data_ptr(), m, k, k, 1, native.KM_BF16, None, q8buf.data_ptr(), sbuf.data_ptr(), stream)
+
+    quant8_rotated()
+    rotate_then_quant8()
+    qr = event_ms(quant8_rotated, reps)
+    q2 = event_ms(rotate_then_quant8, reps)
     out["int8_compute_M16384_K3072_N9216"] = {
         "quant_rows_us": qt * 1e3, "quant_rows_GBps": (m * k * 3 + m * 4) / qt / 1e6, "hbm_peak_GBps": HBM_PEAK_GBS,
         "gemm_ms": gt, "gemm_TOPs": flop / gt / 1e9, "step_ms": st, "step_TOPs": flop / st / 1e9, "peak_TOPs": 5000.0,
+        "rotating_quant_rows_us": qr * 1e3, "rotation_then_quant_rows_us": q2 * 1e3,
+        "rotation_share_of_rotated_fwd": max(qr - qt, 0.0) / (st + max(qr - qt, 0.0)),
+        "rotation_share_of_rotated_fwd_two_kernels": (q2 - qt) / (st + q2 - qt),
     }
     return out
 
@@ -381,7 +446,7 @@ def same_node(dev, x, w, bias, reps):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=200, help="untimed steps first (about 0.1 s: the card needs that long to reach its sustained clocks)")
     ap.add_argument("--config", type=int, default=-1, help="GEMM tile configuration; -1 times every configuration once, as the tuning table does, and takes the fastest")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -443,10 +508,12 @@ def main():
         achieved = GEMM_FLOP / (gemm_ms * 1e-3) / 1e12
         print(json.dumps({"ms_per_step": ms_per_step, "gemm_ms": gemm_ms, "gemm_TFLOPs": achieved, "frac": achieved / FP8_PEAK_TFLOPS, "gemm_tile_config": config, "gemm_tile_configs_ms": tried}))
         return
-    rows_ms = event_ms(lambda: native.quant_mx(x), max(args.steps, 10))
-    fused_rows_ms = event_ms(lambda: native.quant_mx(x, natural=False, packed=True), max(args.steps, 10))
+    ceiling = mfma_ceiling(xq0, wq)
+    qreps = min(max(args.steps, 10), 100)
+    rows_ms = event_ms(lambda: native.quant_mx(x), qreps)
+    fused_rows_ms = event_ms(lambda: native.quant_mx(x, natural=False, packed=True), qreps)
     xt = x.t()
-    cols_ms = event_ms(lambda: native.quant_mx(xt), max(args.steps, 10))
+    cols_ms = event_ms(lambda: native.quant_mx(xt), qreps)
     # the same two kernels on a ring of five input tensors whose outputs are kept alive
     # (760 MB in all, three times the last-level cache): every byte comes from and goes to HBM
     ring = [x] + [torch.randn(M, K, device=dev, dtype=torch.bfloat16) for _ in range(4)]
@@ -461,8 +528,8 @@ def main():
 
     for f in (cold(lambda t: t), cold(lambda t: t.t())):
         event_ms(f, 10)
-    rows_cold_ms = event_ms(cold(lambda t: t), max(args.steps, 10))
-    cols_cold_ms = event_ms(cold(lambda t: t.t()), max(args.steps, 10))
+    rows_cold_ms = event_ms(cold(lambda t: t), qreps)
+    cols_cold_ms = event_ms(cold(lambda t: t.t()), qreps)
     # what a plain device copy of the same number of bytes takes on the same ring: the ceiling a
     # streaming kernel can reach on this card (a copy moves QUANT_BYTES / 1.5 * 2 bytes per call of
     # bf16 in and out; scaled to the quantizer's byte count)
@@ -473,7 +540,7 @@ def main():
         copies[i].copy_(ring[i])
 
     event_ms(cold_copy, 10)
-    copy_cold_ms = event_ms(cold_copy, max(args.steps, 10))
+    copy_cold_ms = event_ms(cold_copy, qreps)
     copy_bytes = 2 * ring[0].numel() * 2
     copy_GBps = copy_bytes / (copy_cold_ms * 1e-3) / 1e9
     del ring, held, copies
@@ -504,38 +571,43 @@ def main():
             "peak": FP8_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / FP8_PEAK_TFLOPS,
-            "traffic": GEMM_TRAFFIC_BYTES,
+            "traffic": profiled_traffic_bytes(),
+            "traffic_source": "profiles/" + os.path.basename(TRAFFIC_PROFILE),
             "algorithmic_flop": GEMM_FLOP,
             "ms": gemm_ms,
+            "peak_sustained": ceiling["TFLOPs"],
+            "frac_of_sustained": achieved / ceiling["TFLOPs"],
+            "sustained": ceiling,
         },
         "quantizer": {
             "bound": "hbm",
             "bytes_per_launch": QUANT_BYTES,
-            "rows_ms": rows_ms,
-            "rows_packed_scales_ms": fused_rows_ms,
-            "rows_GBps": QUANT_BYTES / (rows_ms * 1e-3) / 1e9,
-            "rows_frac": QUANT_BYTES / (rows_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "cols_ms": cols_ms,
-            "cols_GBps": QUANT_BYTES / (cols_ms * 1e-3) / 1e9,
-            "cols_frac": QUANT_BYTES / (cols_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "rows_cold_ms": rows_cold_ms,
-            "rows_cold_GBps": QUANT_BYTES / (rows_cold_ms * 1e-3) / 1e9,
-            "rows_cold_frac": QUANT_BYTES / (rows_cold_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "cols_cold_ms": cols_cold_ms,
-            "cols_cold_GBps": QUANT_BYTES / (cols_cold_ms * 1e-3) / 1e9,
-            "cols_cold_frac": QUANT_BYTES / (cols_cold_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "rows_ms": rows_cold_ms,
+            "rows_GBps": QUANT_BYTES / (rows_cold_ms * 1e-3) / 1e9,
+            "rows_frac": QUANT_BYTES / (rows_cold_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "cols_ms": cols_cold_ms,
+            "cols_GBps": QUANT_BYTES / (cols_cold_ms * 1e-3) / 1e9,
+            "cols_frac": QUANT_BYTES / (cols_cold_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "rows_warm_ms": rows_ms,
+            "rows_warm_packed_scales_ms": fused_rows_ms,
+            "rows_warm_GBps": QUANT_BYTES / (rows_ms * 1e-3) / 1e9,
+            "rows_warm_frac": QUANT_BYTES / (rows_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "cols_warm_ms": cols_ms,
+            "cols_warm_GBps": QUANT_BYTES / (cols_ms * 1e-3) / 1e9,
+            "cols_warm_frac": QUANT_BYTES / (cols_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "copy_cold_ms": copy_cold_ms,
             "copy_cold_GBps": copy_GBps,
             "copy_cold_frac": copy_GBps / HBM_PEAK_GBS,
             "rows_cold_vs_copy": (QUANT_BYTES / (rows_cold_ms * 1e-3) / 1e9) / copy_GBps,
             "cols_cold_vs_copy": (QUANT_BYTES / (cols_cold_ms * 1e-3) / 1e9) / copy_GBps,
-            "note": "rows_/cols_: back-to-back launches on one tensor (the reference's timing method; part of it stays in the 256 MB last-level cache); *_cold_: a ring of tensors larger than that cache; copy_cold_: torch's device copy of one ring tensor (read + write), the practical HBM ceiling of a streaming kernel here",
+            "note": "rows_/cols_: every launch on another tensor of a ring larger than the 256 MB last-level cache, outputs kept alive (every byte from and to HBM); *_warm_: back-to-back launches on one tensor (the reference's timing method; part of it stays in that cache); copy_cold_: torch's device copy of one ring tensor (read + write) on the same ring, the practical HBM ceiling of a streaming kernel here",
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
         },
     }
-    line["same_node"] = same_node(dev, x, w, bias, max(args.steps // 2, 5))
-    line["other_configs"] = other_configs(dev, max(args.steps // 2, 5))
+    reps = min(max(args.steps // 2, 5), 50)
+    line["same_node"] = same_node(dev, x, w, bias, reps)
+    line["other_configs"] = other_configs(dev, reps)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(x, wq, ws, bias)
     print(json.dumps(line))

@@ -94,6 +94,16 @@ int km_quant_blocks(const void *x, int64_t rows, int64_t cols, int64_t stride_ro
 int km_quant_rows_i8(const void *x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,
                      int dtype, const float *col_scale, void *q, float *scale_out, void *stream);
 
+/* The same quantizer over the rotated activation, in one pass over x:
+ * q, scale_out = quantize_rows(group_hadamard(x, group)), the rotation's result rounded to the
+ * 16-bit type before it is quantized, exactly as km_group_hadamard followed by km_quant_rows_i8
+ * gives it. Unit column stride, group >= 16, cols % group == 0, cols <= 4096, x and q 16-byte
+ * aligned, stride_row % 8 == 0 (KM_ERR_UNSUPPORTED otherwise: run the two entry points instead). Replaces
+ * the rotating form (G > 0) of the Triton row quantizer _quant_rows
+ * (src/kohakumoss_kernels/backends/triton/int8.py:47-75). */
+int km_quant_rows_i8_rotated(const void *x, int64_t rows, int64_t cols, int64_t stride_row, int dtype,
+                             int group, void *q, float *scale_out, void *stream);
+
 /* C[M,N] = (A .* 2^(a_scale-127)) (B .* 2^(b_scale-127))^T + bias, A [M,K] and B [N,K] e4m3fn
  * row-major (K contiguous), scales E8M0 bytes, both in the layout scale_layout names
  * (KM_SCALES_ROWMAJOR: [M,K/32] / [N,K/32]; KM_SCALES_PACKED: see km_scales_pack), fp32 accumulation

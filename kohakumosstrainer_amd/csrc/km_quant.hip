@@ -19,6 +19,7 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
+#include "km_hadamard_common.h"
 #include "km_internal.h"
 #include "km_numeric.h"
 #include "km_quant_common.h"
@@ -315,47 +316,62 @@ __global__ __launch_bounds__(256) void scales_pack(const uint8_t* __restrict__ i
 // ---- per-tensor recipe -----------------------------------------------------------------------
 __global__ void fill_u32(uint32_t* p, uint32_t v) { *p = v; }
 
-constexpr int kTensorBlocks = 2048;  // grid-stride: 8 workgroups per compute unit, one atomic each
+// The abs-max pass ends in atomics on one address, and those are served one at a time, about 10 ns
+// each, while the wavefronts that issued them keep their slots: 2048 work-groups of 256 threads cost
+// 19 us in atomics on top of 16 us of reading (6144 work-groups: 61 us). So the pass runs few, large
+// work-groups (two per compute unit, 1024 threads, four 128-bit loads in flight per thread), and a
+// work-group first looks at the value with a plain load and skips the atomic when it cannot raise it.
+constexpr int kAmaxThreads = 1024;
+constexpr int kAmaxBlocks = 512;
+constexpr int kAmaxPiece = kAmaxThreads * 4;  // 128-bit chunks per work-group and trip (64 KiB)
+constexpr int kTensorBlocks = 1 << 20;        // the cast pass: one 16 KiB piece per work-group, grid-stride beyond
 
 // non-negative floats order like their bits: an unsigned atomic max of fp32 bits is an abs-max
 // (NaN patterns stay above infinity)
 template <int DT>
-__global__ __launch_bounds__(256) void tensor_amax(const uint16_t* __restrict__ x, int64_t sr,
-                                                   int64_t sc, int64_t rows, int64_t cols,
-                                                   uint32_t* __restrict__ amax_bits) {
+__global__ __launch_bounds__(kAmaxThreads) void tensor_amax(const uint16_t* __restrict__ x, int64_t sr,
+                                                            int64_t sc, int64_t rows, int64_t cols,
+                                                            uint32_t* __restrict__ amax_bits) {
+  constexpr int T = kAmaxThreads;
   const int64_t n = rows * cols;
   const bool dense = sc == 1 && sr == cols;
   uint32_t m16 = 0;
-  const int64_t stride = (int64_t)gridDim.x * 256;
   if (dense && (cols % 8) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    // a work-group reads whole pieces (four consecutive runs of 16 KiB, one per load of a thread)
     const uint4* src = reinterpret_cast<const uint4*>(x);
     const int64_t nch = n / 8;
-    int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    for (; g + 3 * stride < nch; g += 4 * stride) {
-      const uint4 r0 = src[g], r1 = src[g + stride], r2 = src[g + 2 * stride], r3 = src[g + 3 * stride];
-      const uint32_t a = amax16x8(r0), b = amax16x8(r1), c = amax16x8(r2), d = amax16x8(r3);
-      const uint32_t ab = a > b ? a : b, cd = c > d ? c : d, abcd = ab > cd ? ab : cd;
-      m16 = abcd > m16 ? abcd : m16;
-    }
-    for (; g < nch; g += stride) {
-      const uint32_t a = amax16x8(src[g]);
-      m16 = a > m16 ? a : m16;
+    for (int64_t base = (int64_t)blockIdx.x * kAmaxPiece; base < nch; base += (int64_t)gridDim.x * kAmaxPiece) {
+      const int64_t g = base + threadIdx.x;
+      if (base + kAmaxPiece <= nch) {
+        const uint4 r0 = src[g], r1 = src[g + T], r2 = src[g + 2 * T], r3 = src[g + 3 * T];
+        const uint32_t a = amax16x8(r0), b = amax16x8(r1), c = amax16x8(r2), d = amax16x8(r3);
+        const uint32_t ab = a > b ? a : b, cd = c > d ? c : d, abcd = ab > cd ? ab : cd;
+        m16 = abcd > m16 ? abcd : m16;
+      } else {
+        for (int64_t i = g; i < nch; i += T) {
+          const uint32_t a = amax16x8(src[i]);
+          m16 = a > m16 ? a : m16;
+        }
+      }
     }
   } else {
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    const int64_t stride = (int64_t)gridDim.x * T;
+    for (int64_t i = (int64_t)blockIdx.x * T + threadIdx.x; i < n; i += stride) {
       const int64_t r = i / cols, c = i - r * cols;
       const uint32_t a = x[r * sr + c * sc] & 0x7FFFu;
       m16 = a > m16 ? a : m16;
     }
   }
-  __shared__ uint32_t wave_m[4];
+  __shared__ uint32_t wave_m[T / 64];
   const uint32_t m = wave_max(m16);
   if ((threadIdx.x & 63) == 0) wave_m[threadIdx.x >> 6] = m;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    const uint32_t a = wave_m[0] > wave_m[1] ? wave_m[0] : wave_m[1], b = wave_m[2] > wave_m[3] ? wave_m[2] : wave_m[3];
-    const uint32_t bits = widen_bits<DT>(a > b ? a : b);
-    if (bits != 0) atomicMax(amax_bits, bits);
+  if (threadIdx.x < 64) {
+    const uint32_t mine = threadIdx.x < T / 64 ? wave_m[threadIdx.x] : 0u;
+    const uint32_t bits = widen_bits<DT>(wave_max(mine));
+    // the value only ever grows: a (possibly stale) reading at or above this work-group's maximum
+    // means the atomic could not change it
+    if (threadIdx.x == 0 && bits != 0 && bits > __hip_atomic_load(amax_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(amax_bits, bits);
   }
 }
 
@@ -378,15 +394,19 @@ __global__ __launch_bounds__(256) void tensor_cast(const uint16_t* __restrict__ 
     const uint4* src = reinterpret_cast<const uint4*>(x);
     uint2* dst = reinterpret_cast<uint2*>(q);
     const int64_t nch = n / 8;
-    int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    for (; g + 3 * stride < nch; g += 4 * stride) {
-      const uint4 r0 = src[g], r1 = src[g + stride], r2 = src[g + 2 * stride], r3 = src[g + 3 * stride];
-      dst[g] = divided_codes8<DT>(r0, s, rcp, finite, nan_all);
-      dst[g + stride] = divided_codes8<DT>(r1, s, rcp, finite, nan_all);
-      dst[g + 2 * stride] = divided_codes8<DT>(r2, s, rcp, finite, nan_all);
-      dst[g + 3 * stride] = divided_codes8<DT>(r3, s, rcp, finite, nan_all);
+    // whole 16 KiB pieces per work-group, as in the abs-max pass
+    for (int64_t base = (int64_t)blockIdx.x * 1024; base < nch; base += (int64_t)gridDim.x * 1024) {
+      const int64_t g = base + threadIdx.x;
+      if (base + 1024 <= nch) {
+        const uint4 r0 = src[g], r1 = src[g + 256], r2 = src[g + 512], r3 = src[g + 768];
+        dst[g] = divided_codes8<DT>(r0, s, rcp, finite, nan_all);
+        dst[g + 256] = divided_codes8<DT>(r1, s, rcp, finite, nan_all);
+        dst[g + 512] = divided_codes8<DT>(r2, s, rcp, finite, nan_all);
+        dst[g + 768] = divided_codes8<DT>(r3, s, rcp, finite, nan_all);
+      } else {
+        for (int64_t i = g; i < nch; i += 256) dst[i] = divided_codes8<DT>(src[i], s, rcp, finite, nan_all);
+      }
     }
-    for (; g < nch; g += stride) dst[g] = divided_codes8<DT>(src[g], s, rcp, finite, nan_all);
   } else {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
       const int64_t r = i / cols, c = i - r * cols;
@@ -596,6 +616,120 @@ __global__ __launch_bounds__(256) void quant_i8_rows_generic(const uint16_t* __r
     if (col_scale != nullptr) v *= col_scale[c];
     dst[c] = (uint8_t)i8_code(v, s);
   }
+}
+
+// ---- int8 per-row quantizer of a rotated activation ---------------------------------------------
+// q, s = quantize_rows(group_hadamard(x, G)) in one pass over x (the reference's Triton quantizer
+// rotates the tile it has loaded, backends/triton/int8.py:47-75). A work-group owns one row of up to
+// 4096 elements: it widens the row into LDS and runs the butterfly stages of km_hadamard.hip there
+// (same stages, same order, the same rounding to the 16-bit type at the end: the rotated values are
+// those the rotation kernel would have written). The last double pass leaves a lane with 16
+// consecutive rotated elements in registers; the row's abs-max is joined over the work-group and the
+// lane writes its 16 codes with one 128-bit store: the rotated row never goes back to LDS or memory.
+// Groups of 16 and more (a group of 4 has no double pass; it takes the two kernels).
+constexpr int kRotMaxCols = 4096;
+
+template <int DT, int J>
+__global__ __launch_bounds__(256) void rotate_quant_i8_rows(const uint16_t* __restrict__ x, int64_t ld, uint32_t cols,
+                                                            uint8_t* __restrict__ q, float* __restrict__ scale) {
+  static_assert(J >= 2, "the last stages run as a double pass");
+  constexpr int G = 1 << (2 * J);
+  constexpr float kScale = 1.0f / (float)(1 << J);
+  __shared__ __attribute__((aligned(16))) float tile[kRotMaxCols];
+  __shared__ uint32_t wave_m[4];
+  const uint32_t t = threadIdx.x, row = blockIdx.x;
+  const uint32_t chunks = cols / 8, units = cols / 16;
+  const uint4* src = reinterpret_cast<const uint4*>(x + (uint64_t)row * (uint64_t)ld);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const uint32_t c = t + 256 * i;
+    if (c < chunks) {
+      float f[8];
+      widen8<DT>(src[c], f);
+      *reinterpret_cast<float4*>(&tile[c * 8]) = make_float4(f[0], f[1], f[2], f[3]);
+      *reinterpret_cast<float4*>(&tile[c * 8 + 4]) = make_float4(f[4], f[5], f[6], f[7]);
+    }
+  }
+  __syncthreads();
+  if constexpr (J % 2 == 1) {
+    constexpr uint32_t S1 = G / 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t qd = t + 256 * i;
+      if (qd < cols / 4) {
+        const uint32_t first = (qd / S1) * 4 * S1 + qd % S1;
+        float v0 = tile[first], v1 = tile[first + S1], v2 = tile[first + 2 * S1], v3 = tile[first + 3 * S1];
+        h4(v0, v1, v2, v3);
+        tile[first] = v0; tile[first + S1] = v1; tile[first + 2 * S1] = v2; tile[first + 3 * S1] = v3;
+      }
+    }
+    __syncthreads();
+  }
+  constexpr int kDouble = J / 2;
+  constexpr uint32_t kRest = J % 2 == 1 ? G / 4 : G;
+  float v[4][4];
+  const bool active = t < units;
+#pragma unroll
+  for (int p = 0; p < kDouble; ++p) {
+    const uint32_t S = kRest >> (4 * (p + 1));
+    const uint32_t first = (t / S) * 16 * S + t % S;
+    if (active) {
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) v[a][b] = tile[first + (4 * a + b) * S];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) h4(v[0][b], v[1][b], v[2][b], v[3][b]);
+#pragma unroll
+      for (int a = 0; a < 4; ++a) h4(v[a][0], v[a][1], v[a][2], v[a][3]);
+    }
+    if (p < kDouble - 1) {
+      if (active) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+          for (int b = 0; b < 4; ++b) tile[first + (4 * a + b) * S] = v[a][b];
+      }
+      __syncthreads();
+    }
+  }
+  // lane t holds elements [16 t, 16 t + 16) of the rotated row: round them as the rotation kernel
+  // stores them, join the abs-max, quantize
+  uint32_t m = 0;
+  if (active) {
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        v[a][b] = had_widen<DT>(had_narrow<DT>(v[a][b] * kScale));
+        const uint32_t bits = f32_bits(v[a][b]) & kAbsMask;
+        m = bits > m ? bits : m;
+      }
+  }
+  m = wave_max(m);
+  if ((t & 63) == 0) wave_m[t >> 6] = m;
+  __syncthreads();
+  {
+    const uint32_t m01 = wave_m[0] > wave_m[1] ? wave_m[0] : wave_m[1], m23 = wave_m[2] > wave_m[3] ? wave_m[2] : wave_m[3];
+    m = m01 > m23 ? m01 : m23;
+  }
+  const float s = i8_scale_of(m);
+  if (t == 0) scale[row] = s;
+  if (!active) return;
+  // the rotated values are 16-bit patterns at or below the row's amax: the quotient comes from the
+  // rounded reciprocal and two fused corrections, as in quant_i8_rows; a row with an infinite amax divides
+  const bool fast = m < kInfBits;
+  const float rcp = __fdiv_rn(1.0f, s);
+  uint32_t packed[4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    uint32_t b4[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+      b4[b] = fast ? ((uint32_t)(int)__builtin_amdgcn_fmed3f(__builtin_rintf(quotient(v[a][b], s, rcp)), -127.0f, 127.0f) & 0xFFu) : i8_code(v[a][b], s);
+    packed[a] = b4[0] | (b4[1] << 8) | (b4[2] << 16) | (b4[3] << 24);
+  }
+  *reinterpret_cast<uint4*>(q + (uint64_t)row * cols + 16 * t) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
 }
 
 // ---- block recipe: fp32 scales per 128 columns (activations) or per 128 x 128 block (weights) ----
@@ -820,11 +954,13 @@ extern "C" int km_quant_tensor(const void* x, int64_t rows, int64_t cols, int64_
   const int64_t n = rows * cols;
   if (n > 0 && (!x || !q)) return km_fail(KM_ERR_ARG, "km_quant_tensor: null pointer");
   hipLaunchKernelGGL(fill_u32, dim3(1), dim3(1), 0, st, amax_workspace, 0u);
-  int64_t want = (n / 8 + 255) / 256;
+  int64_t want = (n / 8 + 1023) / 1024;  // one 16 KiB piece per work-group and trip
   unsigned blocks = (unsigned)(want < 1 ? 1 : (want > kTensorBlocks ? kTensorBlocks : want));
+  const int64_t amax_want = (n / 8 + kAmaxPiece - 1) / kAmaxPiece;
+  const unsigned amax_blocks = (unsigned)(amax_want < 1 ? 1 : (amax_want > kAmaxBlocks ? kAmaxBlocks : amax_want));
   const uint16_t* xp = (const uint16_t*)x;
   KM_DISPATCH_DT(dtype, {
-    if (n > 0) hipLaunchKernelGGL(tensor_amax<DT>, dim3(blocks), dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, amax_workspace);
+    if (n > 0) hipLaunchKernelGGL(tensor_amax<DT>, dim3(amax_blocks), dim3(kAmaxThreads), 0, st, xp, stride_row, stride_col, rows, cols, amax_workspace);
     hipLaunchKernelGGL(tensor_cast<DT>, dim3(blocks), dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, amax_workspace, (uint8_t*)q, scale_out);
   });
   return km_check_launch("km_quant_tensor");
@@ -929,4 +1065,33 @@ extern "C" int km_quant_rows_i8(const void* x, int64_t rows, int64_t cols, int64
                                              (uint32_t)rows, cols, col_scale, (uint8_t*)q, scale_out));
   }
   return km_check_launch("km_quant_rows_i8");
+}
+
+extern "C" int km_quant_rows_i8_rotated(const void* x, int64_t rows, int64_t cols, int64_t stride_row, int dtype, int group,
+                                        void* q, float* scale_out, void* stream) {
+  if (dtype != KM_BF16 && dtype != KM_F16) return km_fail(KM_ERR_ARG, "km_quant_rows_i8_rotated: dtype must be bf16 or f16");
+  int stages = 0;
+  for (int g = group; g > 1 && g % 4 == 0; g /= 4) ++stages;
+  if (group < 4 || (1 << (2 * stages)) != group || stages > 5)
+    return km_fail(KM_ERR_ARG, "km_quant_rows_i8_rotated: group must be 4, 16, 64, 256 or 1024");
+  if (rows < 0 || cols < 0 || cols % group) return km_fail(KM_ERR_ARG, "km_quant_rows_i8_rotated: cols must be a non-negative multiple of the group");
+  if (rows == 0 || cols == 0) return KM_OK;
+  if (rows > 0x7FFFFFFFll) return km_fail(KM_ERR_ARG, "km_quant_rows_i8_rotated: too many rows");
+  if (!x || !q || !scale_out) return km_fail(KM_ERR_ARG, "km_quant_rows_i8_rotated: null pointer");
+  if (group < 16 || cols > kRotMaxCols || stride_row % 8 || stride_row < cols || (reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(q) & 15))
+    return km_fail(KM_ERR_UNSUPPORTED, "km_quant_rows_i8_rotated: groups of 16 and more, rows of up to 4096 elements, 16-byte aligned operands, row stride a multiple of 8");
+  hipStream_t st = (hipStream_t)stream;
+  const uint16_t* xp = (const uint16_t*)x;
+  const dim3 grid((unsigned)rows);
+#define KM_ROT_CASE(J) hipLaunchKernelGGL((rotate_quant_i8_rows<DT, J>), grid, dim3(256), 0, st, xp, stride_row, (uint32_t)cols, (uint8_t*)q, scale_out)
+  KM_DISPATCH_DT(dtype, {
+    switch (stages) {
+      case 2: KM_ROT_CASE(2); break;
+      case 3: KM_ROT_CASE(3); break;
+      case 4: KM_ROT_CASE(4); break;
+      default: KM_ROT_CASE(5); break;
+    }
+  });
+#undef KM_ROT_CASE
+  return km_check_launch("km_quant_rows_i8_rotated");
 }

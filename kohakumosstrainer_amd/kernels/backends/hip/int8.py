@@ -2,10 +2,14 @@
 int32 MFMA with both scales and the bias applied to the accumulator in the eager path's order of
 roundings (outputs equal the eager reference bit for bit), and the two input-gradient modes.
 Host-side counterpart of reference `backends/triton/int8.py` (launchers :234-270, registration
-:273-281). A rotated base (`group` > 0) gets one pass of the HIP butterfly kernel over x before
-the quantizer and one over dx. The int8 input gradient contracts over N, so it reads a `[K, N]` copy of the codes,
-made per call as the reference makes its column-major copy (`int8/formats.py:55-58`).
+:273-281). A rotated base (`group` > 0) has its activations rotated inside the quantizer kernel
+(rows of up to 4096 elements; longer rows get a pass of the butterfly kernel first) and one pass of
+the butterfly kernel over dx. The int8 input gradient contracts over N, so it reads a `[K, N]` copy
+of the codes; the reference makes its column-major copy per call (`int8/formats.py:55-58`), here it
+is made once per frozen code tensor and kept for as long as that tensor lives.
 """
+
+import weakref
 
 from kohakumosstrainer_amd import native
 from kohakumosstrainer_amd.kernels import registry, tuning
@@ -44,12 +48,27 @@ def _pick(kernel, kind, m, n, k, a, bias, launch, in_backward):
     return cfg
 
 
+# `[K, N]` copies of frozen `[N, K]` code tensors, by the identity of the tensor object. An entry goes
+# when its tensor is collected and is remade when the tensor has been written to since.
+_TRANSPOSED: dict[int, tuple] = {}
+
+
+def transposed_codes(q):
+    key = id(q)
+    hit = _TRANSPOSED.get(key)
+    if hit is not None and hit[0]() is q and hit[1] == q._version:
+        return hit[2]
+    q_t = q.t().contiguous()
+    _TRANSPOSED[key] = (weakref.ref(q, lambda _ref, key=key: _TRANSPOSED.pop(key, None)), q._version, q_t)
+    return q_t
+
+
 def fwd(x, q, scale, bias, group):
     m, k = x.shape
     n = q.shape[0]
     _check("fwd", k)
     q, scale = q.contiguous(), scale.float().contiguous()
-    xq, xs = native.quant_rows_i8(rotate_2d(x, group) if group else x)
+    xq, xs = native.quant_rows_i8_rotated(x, group) if group else native.quant_rows_i8(x)
     cfg = _pick("int8_fwd", "fwd", m, n, k, x, bias, lambda c: lambda: native.gemm_i8_rows(xq, xs, q, scale, bias, x.dtype, c["id"]), False)
     return native.gemm_i8_rows(xq, xs, q, scale, bias, x.dtype, cfg["id"])
 
@@ -62,7 +81,7 @@ def dgrad(dy, q, scale, group, mode):
         return rotate_2d(dx, group) if group else dx
     _check("dgrad", n)
     gq, gs = native.quant_rows_i8(dy, scale)
-    q_t = q.t().contiguous()
+    q_t = transposed_codes(q)
     cfg = _pick("int8_dgrad", "dgrad", m, k, n, dy, None, lambda c: lambda: native.gemm_i8_rows(gq, gs, q_t, None, None, dy.dtype, c["id"]), True)
     dx = native.gemm_i8_rows(gq, gs, q_t, None, None, dy.dtype, cfg["id"])
     return rotate_2d(dx, group) if group else dx

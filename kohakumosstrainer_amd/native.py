@@ -36,6 +36,7 @@ EXPORTS = (
     "km_quant_rows",
     "km_quant_blocks",
     "km_quant_rows_i8",
+    "km_quant_rows_i8_rotated",
     "km_gemm_mx",
     "km_gemm_mx_fused",
     "km_gemm_fp8_rows_fused",
@@ -78,6 +79,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.km_quant_rows.argtypes = [p, i64, i64, i64, i64, i32, p, p, p]
     lib.km_quant_blocks.argtypes = [p, i64, i64, i64, i64, i32, i32, p, p, p, p]
     lib.km_quant_rows_i8.argtypes = [p, i64, i64, i64, i64, i32, p, p, p, p]
+    lib.km_quant_rows_i8_rotated.argtypes = [p, i64, i64, i64, i32, i32, p, p, p]
     lib.km_gemm_mx.argtypes = [p, p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_gemm_mx_fused.argtypes = [p, i64, p, p, p, p, i64, i64, i64, i32, p]
     lib.km_gemm_fp8_rows_fused.argtypes = [p, i64, p, p, p, p, i64, i64, i64, i32, p]
@@ -293,6 +295,27 @@ def quant_rows_i8(x: Tensor, col_scale: Tensor | None = None) -> tuple[Tensor, T
     s = torch.empty(rows, device=x.device, dtype=torch.float32)
     with torch.cuda.device(x.device):
         _check(load().km_quant_rows_i8(x.data_ptr(), rows, k, x.stride(0), x.stride(1), _dtype_code(x.dtype), None if col_scale is None else col_scale.data_ptr(), q.data_ptr(), s.data_ptr(), _stream(x)))
+    return q, s
+
+
+ROTATED_QUANT_MAX_COLS = 4096  # longest row the rotating int8 quantizer holds in LDS (four rows of fp32)
+
+
+def quant_rows_i8_rotated(x: Tensor, group: int) -> tuple[Tensor, Tensor]:
+    """`quant_rows_i8(group_hadamard(x, group))`, bit for bit: one kernel that rotates the rows in
+    LDS on their way to the quantizer where the rows fit (groups of 16 and more, unit-stride rows of
+    up to `ROTATED_QUANT_MAX_COLS` elements), the two kernels one after the other elsewhere."""
+    if x.dim() != 2:
+        raise ValueError(f"int8 operand must be 2-D, got {tuple(x.shape)}")
+    _on_gpu(x)
+    rows, k = x.shape
+    fits = group >= 16 and x.stride(1) == 1 and k <= ROTATED_QUANT_MAX_COLS and x.stride(0) % 8 == 0 and x.stride(0) >= k and x.data_ptr() % 16 == 0
+    if not fits or rows == 0:
+        return quant_rows_i8(group_hadamard(x, group))
+    q = torch.empty(rows, k, device=x.device, dtype=torch.int8)
+    s = torch.empty(rows, device=x.device, dtype=torch.float32)
+    with torch.cuda.device(x.device):
+        _check(load().km_quant_rows_i8_rotated(x.data_ptr(), rows, k, x.stride(0), _dtype_code(x.dtype), int(group), q.data_ptr(), s.data_ptr(), _stream(x)))
     return q, s
 
 

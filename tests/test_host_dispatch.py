@@ -60,6 +60,117 @@ def test_fallback_walks_priority_and_rebinds_siblings(fake_ops):
     assert c.backend == "second", "a backend that failed here is skipped at the next resolve"
 
 
+class _FailsInBackward(torch.autograd.Function):
+    """A backend whose forward is fine and whose backward cannot launch."""
+
+    @staticmethod
+    def forward(ctx, x, w):
+        ctx.save_for_backward(x, w)
+        return x @ w.t()
+
+    @staticmethod
+    def backward(ctx, g):
+        raise BackendUnavailable("fake_linear", {"dgrad": "kernel does not build"})
+
+
+@pytest.fixture
+def backward_failure():
+    registry.load_backends()
+    calls = []
+
+    def hip(x, w):
+        calls.append("hip")
+        return _FailsInBackward.apply(x, w)
+
+    def eager(x, w):
+        calls.append("eager")
+        return x @ w.t()
+
+    registry.register("fake_linear", "hip", hip)
+    registry.register("fake_linear", "eager", eager)
+    registry.set_priority("cpu", ("hip", "eager"))
+    yield calls
+    registry.reset_priority()
+    registry.clear_failures()
+    registry.forget_disk_failures()
+    registry.unregister("fake_linear")
+
+
+def test_failure_inside_backward_moves_on_and_recomputes(backward_failure):
+    """Reference `registry.py:280-314`: the backend fails only in backward; the op and its sibling
+    move to the next backend and the gradients come from a second forward + backward there."""
+    op = registry.resolve("fake_linear", "cpu", torch.float32)
+    sibling = registry.resolve("fake_linear", "cpu", torch.float32)
+    assert op.backend == "hip" and op.guard, "an op with somewhere to go runs its backward under guard"
+    x = torch.randn(5, 8, requires_grad=True)
+    w = torch.randn(3, 8, requires_grad=True)
+    y = op(x, w)
+    assert op.backend == "hip" and backward_failure == ["hip"]
+    g = torch.randn(5, 3)
+    y.backward(g)
+    assert op.backend == "eager" and sibling.backend == "eager", "the sibling moves with it"
+    assert backward_failure == ["hip", "eager"], "forward ran again through the next backend"
+    assert torch.allclose(x.grad, g @ w.detach()) and torch.allclose(w.grad, g.t() @ x.detach())
+    assert torch.equal(y.detach(), x.detach() @ w.detach().t())
+    assert not op.guard, "the last backend of the chain has nothing to give way to"
+    assert any(k[0] == "fake_linear" and k[1] == "hip" for k in registry.failures())
+    # without grad nothing is guarded, and the next call goes straight to the backend that works
+    with torch.no_grad():
+        op(x, w)
+    assert backward_failure == ["hip", "eager", "eager"]
+
+
+def test_guard_refuses_inputs_written_between_forward_and_backward(backward_failure):
+    op = registry.resolve("fake_linear", "cpu", torch.float32)
+    x = torch.randn(5, 8, requires_grad=True)
+    w = torch.randn(3, 8)
+    y = op(x, w)
+    w.add_(1.0)  # the recompute would see another weight: autograd's version check must refuse
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        y.backward(torch.ones(5, 3))
+
+
+def test_settle_guards_and_exercise(backward_failure):
+    registry.unregister("fake_linear", "hip")
+    registry.register("fake_linear", "hip", lambda x, w: x @ w.t())  # a backend that works
+    op = registry.resolve("fake_linear", "cpu", torch.float32)
+    x = torch.randn(2, 8, requires_grad=True)
+    w = torch.randn(3, 8)
+    assert op.guard
+    op(x, w).sum().backward()
+    assert op.guard, "proven, but the guard is lifted only at a step boundary"
+    assert registry.settle_guards() == 1 and not op.guard and op.backend == "hip"
+    op(x, w).sum().backward()  # the plain path
+    other = registry.resolve("fake_linear", "cpu", torch.float16)
+    ran = registry.exercise(other, lambda o: o(x.detach().half().requires_grad_(True), w.half()).sum().backward())
+    assert ran is None and not other.guard, "a prewarm that went through lifts the guard at once"
+
+
+def test_toolchain_failures_at_build_time_outlive_the_process(backward_failure):
+    """Reference `status.py:111-133`: only a build / toolchain failure met at build time is written
+    to disk; a later process (here: the in-memory state dropped) does not try that backend again."""
+    op = registry.resolve("fake_linear", "cpu", torch.float32)
+    x = torch.randn(2, 8, requires_grad=True)
+    w = torch.randn(3, 8)
+    registry.exercise(op, lambda o: o(x, w).sum().backward())
+    assert op.backend == "eager"
+    registry.clear_failures()
+    registry._S.disk = None  # what a new process starts with: nothing in memory, the file on disk
+    why = registry.available("fake_linear", "cpu", torch.float32)
+    assert why["hip"] is not None and "earlier process" in why["hip"], why
+    assert registry.resolve("fake_linear", "cpu", torch.float32).backend == "eager"
+    assert registry.resolve("fake_linear", "cpu", torch.float16).backend == "hip", "another query is not covered by the record"
+    # a failure in a live call (outside build time) stays in the process
+    registry.forget_disk_failures()
+    live = registry.resolve("fake_linear", "cpu", torch.bfloat16)
+    xb = x.detach().bfloat16().requires_grad_(True)
+    live(xb, w.bfloat16()).sum().backward()
+    assert live.backend == "eager"
+    registry.clear_failures()
+    registry._S.disk = None
+    assert registry.available("fake_linear", "cpu", torch.bfloat16)["hip"] is None
+
+
 def test_pinned_backend_has_no_fallback(fake_ops):
     op = registry.resolve("fake_op", "cpu", torch.float32, backend="hip")
     with pytest.raises(BackendUnavailable):
