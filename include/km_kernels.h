@@ -222,6 +222,19 @@ int km_wo_gemm_dgrad_static(const void *dy, const void *q, const float *scale, v
                             int64_t M, int64_t N, int64_t K, int q_format, int dtype, int config,
                             void *stream);
 
+/* Which kernel class the weight-only entry points above would run for these operands: the tiled MFMA
+ * kernels (KM_PATH_TILED) or the kernel with one thread per output element that serves every other
+ * shape and alignment, correct and far slower (KM_PATH_ELEMENTWISE: K % 8 != 0 in forward; N % 8 != 0,
+ * K % 4 != 0, operands not 16-byte aligned or extreme extents in the input gradient). Pointers are
+ * only inspected for alignment. direction: KM_WO_FWD (a = x, c = y), KM_WO_DGRAD_W16 (a = dy, c = dx),
+ * KM_WO_DGRAD_TRANSPOSED (km_wo_gemm_dgrad and km_wo_gemm_dgrad_static). A host layer uses it to tell
+ * its caller about the slow path instead of timing it silently; no counterpart in the reference,
+ * whose Triton kernels mask ragged tiles. */
+enum { KM_WO_FWD = 0, KM_WO_DGRAD_W16 = 1, KM_WO_DGRAD_TRANSPOSED = 2 };
+enum { KM_PATH_TILED = 0, KM_PATH_ELEMENTWISE = 1 };
+int km_wo_gemm_path(int direction, const void *a, const void *q, const void *scale, const void *c,
+                    int64_t M, int64_t N, int64_t K);
+
 /* Group Hadamard rotation (ConvRot): y[r, :] = x[r, :] . blockdiag(H_group), H_group the normalised
  * Kronecker power of H4 = [[1,1,1,-1],[1,1,-1,1],[1,-1,1,1],[-1,1,1,1]] (symmetric, its own
  * inverse), group in {4, 16, 64, 256, 1024} dividing cols; x and y [rows, cols] contiguous,

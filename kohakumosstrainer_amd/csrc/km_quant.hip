@@ -130,7 +130,9 @@ constexpr int kColsTR = 128;  // rows of x per tile (4 blocks)
 constexpr int kColsTC = 128;  // columns of x per tile: 256-byte row segments
 constexpr int kColsPitch = kColsTC / 2 + 4;  // dwords per staged row (16-byte aligned rows)
 constexpr int kColsHalves = kColsTR / 16;    // half-blocks of 16 rows per tile
-constexpr int kColsSkew = 64 / kColsHalves;  // extra dwords after each 16 rows: a wavefront's reads (8 half-blocks x 8 column pairs) hit 64 banks
+constexpr int kColsSkew = 32 / kColsHalves;  // extra dwords after each 16 rows. LDS serves a 32-bit read 32 lanes and 32 banks at a time: the
+                                             // 8 half-blocks x 4 column pairs of such a half-wavefront hit 32 different banks (a skew of 8, right for 64
+                                             // banks, measured SQ_LDS_BANK_CONFLICT at a third of SQ_LDS_IDX_ACTIVE: two lanes per bank)
 
 // MX: one E8M0 scale per block of 32 rows, found here. !MX: one fp32 scale per column of x (per
 // row of q_t) from `col_amax`, the fp32 bits of each column's amax taken by an earlier pass;

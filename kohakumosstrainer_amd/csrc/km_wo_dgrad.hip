@@ -37,12 +37,7 @@ __global__ __launch_bounds__(256) void wo_dgrad_scalar(const uint16_t* __restric
 template <int DT, int QF, int SK>
 static int dispatch_w16(int config, const void* dy, const void* q, const void* scale, int scale_ld, void* dx, int M, int N,
                         int K, hipStream_t st) {
-  const uintptr_t bits = reinterpret_cast<uintptr_t>(dy) | reinterpret_cast<uintptr_t>(dx);
-  // an empty contraction takes the scalar kernel too: it writes zeros and reads no operand; so does a
-  // q so wide that 32 of its rows pass 2^31 bytes (the tiled kernels step through q by that stride), and a
-  // contraction so long that the 256 rows of dy[M, N] a tile reads pass 2^31 bytes (32-bit offsets
-  // from the tile's first row)
-  if (N == 0 || N % 8 || K % 4 || K > 0x7FFFFFFF / 32 || N > kMaxTiledRowElems || (bits & 15) || (reinterpret_cast<uintptr_t>(q) & 3) || (reinterpret_cast<uintptr_t>(scale) & 3)) {
+  if (!wo_w16_tiles_take(dy, q, scale, dx, N, K)) {
     const int64_t n = (int64_t)M * K;
     hipLaunchKernelGGL((wo_dgrad_scalar<DT, QF, SK>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (const uint16_t*)dy,
                        (const uint8_t*)q, scale, scale_ld, (uint16_t*)dx, M, N, K);

@@ -105,7 +105,7 @@ static int dispatch_wo(int config, const void* a, const void* q, const float* sc
   // The tiles read A through a descriptor based at the tile's first row with 32-bit byte offsets: 256
   // rows of A must stay below 2^31 bytes. The forward's A is capped as a whole; the gradient dy[M, KC]
   // is not, so a very long contraction takes the element-wise kernel.
-  if (KC % 8 || (DGRAD && KC > kMaxTiledRowElems) || ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(q)) & 15)) {
+  if (!wo_tiles_take(DGRAD, a, q, KC)) {
     const int64_t n = (int64_t)M * NO;
     hipLaunchKernelGGL((wo_gemm_scalar<DT, QF, DGRAD>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
                        (const uint16_t*)a, (const uint8_t*)q, scale, (const uint16_t*)bias, (uint16_t*)c, M, NO, KC);
@@ -218,4 +218,13 @@ extern "C" int km_wo_gemm_dgrad_static(const void* dy, const void* q, const floa
   }
   // the transposition rewrites all N*K bytes the GEMM reads, so nothing of an earlier call shows
   return km_wo_gemm_dgrad(dy, q, scale, dx, codes_t, M, N, K, q_format, dtype, config, stream);
+}
+
+extern "C" int km_wo_gemm_path(int direction, const void* a, const void* q, const void* scale, const void* c, int64_t M, int64_t N,
+                               int64_t K) {
+  (void)M;
+  if (direction == KM_WO_FWD) return wo_tiles_take(false, a, q, K) ? KM_PATH_TILED : KM_PATH_ELEMENTWISE;
+  if (direction == KM_WO_DGRAD_W16) return wo_w16_tiles_take(a, q, scale, c, N, K) ? KM_PATH_TILED : KM_PATH_ELEMENTWISE;
+  if (direction == KM_WO_DGRAD_TRANSPOSED) return wo_tiles_take(true, a, q, N) ? KM_PATH_TILED : KM_PATH_ELEMENTWISE;  // q: the transposed codes (the workspace)
+  return km_fail(KM_ERR_ARG, "km_wo_gemm_path: unknown direction");
 }

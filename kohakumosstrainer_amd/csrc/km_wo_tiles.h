@@ -38,6 +38,23 @@ inline int wo_tiles_dgrad_n(int q_format, int scale_kind, int config, const void
 // longest row of a 16-bit operand that a 256-row tile can address with 32-bit byte offsets
 constexpr int kMaxTiledRowElems = 0x7FFFFFFF / (256 * 2);
 
+// Whether a problem runs on the tiled kernels; anything else goes to a kernel with one thread per output
+// element, which is correct for every shape and alignment and far slower. The dispatchers and
+// km_wo_gemm_path() ask the same functions.
+// forward / input gradient over transposed codes: A [M, KC] 16-bit, codes [NO, KC]
+inline bool wo_tiles_take(bool dgrad, const void* a, const void* q, int64_t KC) {
+  return KC % 8 == 0 && !(dgrad && KC > kMaxTiledRowElems) && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(q)) & 15) == 0;
+}
+// input gradient over the codes as stored: dy [M, N], q [N, K], dx [M, K]. An empty contraction takes
+// the element-wise kernel too (it writes zeros and reads no operand); so does a q so wide that 32 of its
+// rows pass 2^31 bytes (the tiled kernels step through q by that stride), and a contraction so long that
+// the 256 rows of dy a tile reads pass 2^31 bytes (32-bit offsets from the tile's first row)
+inline bool wo_w16_tiles_take(const void* dy, const void* q, const void* scale, const void* dx, int64_t N, int64_t K) {
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(dy) | reinterpret_cast<uintptr_t>(dx);
+  return N != 0 && N % 8 == 0 && K % 4 == 0 && K <= 0x7FFFFFFF / 32 && N <= kMaxTiledRowElems && (bits & 15) == 0 &&
+         (reinterpret_cast<uintptr_t>(q) & 3) == 0 && (reinterpret_cast<uintptr_t>(scale) & 3) == 0;
+}
+
 // argument checks shared by the entry points
 int check_wo_args(const char* who, const void* a, const void* q, const void* scale, void* c, int64_t M, int64_t N, int64_t K,
                   int q_format, int dtype, int config);

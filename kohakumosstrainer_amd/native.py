@@ -49,6 +49,7 @@ EXPORTS = (
     "km_wo_gemm_dgrad",
     "km_wo_gemm_dgrad_w16",
     "km_wo_gemm_dgrad_static",
+    "km_wo_gemm_path",
     "km_group_hadamard",
     "km_probe_mfma_ceiling",
     "km_num_configs",
@@ -92,6 +93,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.km_wo_gemm_dgrad.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_wo_gemm_dgrad_w16.argtypes = [p, p, p, i32, i64, p, i64, i64, i64, i32, i32, i32, p]
     lib.km_wo_gemm_dgrad_static.argtypes = [p, p, p, p, i64, i64, i64, i32, i32, i32, p]
+    lib.km_wo_gemm_path.argtypes = [i32, p, p, p, p, i64, i64, i64]
     lib.km_group_hadamard.argtypes = [p, i64, i64, i32, i32, p, p]
     lib.km_probe_mfma_ceiling.argtypes = [p, p, p, i64, i32, c.POINTER(c.c_int64), p]
     lib.km_num_configs.argtypes = [i32]
@@ -554,6 +556,29 @@ def _wo_operands(x: Tensor, q: Tensor, scale: Tensor):
     return x.contiguous(), q.contiguous(), scale.to(torch.float32).contiguous()
 
 
+class SlowPathWarning(UserWarning):
+    """A problem left the tiled kernels for the one-thread-per-element kernel (ragged K or N, or operands
+    that are not 16-byte aligned): correct, and slower by orders of magnitude."""
+
+
+WO_FWD, WO_DGRAD_W16, WO_DGRAD_TRANSPOSED = 0, 1, 2
+_SLOW_SEEN: set[tuple] = set()
+
+
+def _note_path(direction: int, a: Tensor, q: Tensor, scale: Tensor, c: Tensor, m: int, n: int, k: int) -> None:
+    """Warn, once per direction and shape, when the library will serve this problem with its
+    element-wise kernel."""
+    key = (direction, m, n, k)
+    if key in _SLOW_SEEN:
+        return
+    if load().km_wo_gemm_path(direction, a.data_ptr(), q.data_ptr(), scale.data_ptr(), c.data_ptr(), m, n, k) == 1:
+        _SLOW_SEEN.add(key)
+        import warnings
+
+        what = ("forward", "input gradient", "input gradient (transposed codes)")[direction]
+        warnings.warn(f"weight-only {what} M={m} N={n} K={k}: shape or alignment outside the tiled kernels, the element-wise kernel serves it", SlowPathWarning, stacklevel=3)
+
+
 def wo_gemm_fwd(x: Tensor, q: Tensor, scale: Tensor, bias: Tensor | None, config: int = 0) -> Tensor:
     """`(x @ q^T) * scale + bias` -> `[M, N]` in x's dtype; q `[N, K]` int8 / e4m3."""
     x, q, scale = _wo_operands(x, q, scale)
@@ -567,6 +592,7 @@ def wo_gemm_fwd(x: Tensor, q: Tensor, scale: Tensor, bias: Tensor | None, config
         _on_gpu(x, bias)
         bias = bias.to(x.dtype).contiguous()
     y = torch.empty(m, n, device=x.device, dtype=x.dtype)
+    _note_path(WO_FWD, x, q, scale, y, m, n, k)
     with torch.cuda.device(x.device):
         _check(load().km_wo_gemm_fwd(x.data_ptr(), q.data_ptr(), scale.data_ptr(), None if bias is None else bias.data_ptr(), y.data_ptr(), m, n, k, _QFORMATS[q.dtype], _dtype_code(x.dtype), config, _stream(x)))
     return y
@@ -611,6 +637,7 @@ def wo_gemm_dgrad(dy: Tensor, q: Tensor, scale: Tensor, config: int = 0, recipe:
     if q.dtype == torch.int8 and kind != WSCALE_ROWS:
         raise ValueError("int8 codes take one scale per row")
     dx = torch.empty(m, k, device=dy.device, dtype=dy.dtype)
+    _note_path(WO_DGRAD_W16, dy, q, scale, dx, m, n, k)
     with torch.cuda.device(dy.device):
         _check(load().km_wo_gemm_dgrad_w16(dy.data_ptr(), q.data_ptr(), scale.data_ptr(), kind, ld, dx.data_ptr(), m, n, k, _QFORMATS[q.dtype], _dtype_code(dy.dtype), config, _stream(dy)))
     return dx

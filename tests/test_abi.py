@@ -64,6 +64,23 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.km_scales_packed_bytes(100, 96) == -1
 
 
+def test_weight_only_path_query_names_the_slow_kernel():
+    """`km_wo_gemm_path` only looks at extents and pointer alignment: no GPU needed."""
+    lib = native.load()
+    tiled, slow = 0, 1
+    a, q, s, c = 4096, 8192, 1024, 16384  # stand-in addresses, 16-byte aligned
+    assert lib.km_wo_gemm_path(native.WO_FWD, a, q, s, c, 64, 256, 512) == tiled
+    assert lib.km_wo_gemm_path(native.WO_FWD, a, q, s, c, 64, 256, 516) == slow  # K % 8
+    assert lib.km_wo_gemm_path(native.WO_FWD, a + 2, q, s, c, 64, 256, 512) == slow  # alignment
+    assert lib.km_wo_gemm_path(native.WO_DGRAD_W16, a, q, s, c, 64, 256, 512) == tiled
+    assert lib.km_wo_gemm_path(native.WO_DGRAD_W16, a, q, s, c, 64, 250, 512) == slow  # N % 8
+    assert lib.km_wo_gemm_path(native.WO_DGRAD_W16, a, q, s, c, 64, 256, 510) == slow  # K % 4
+    assert lib.km_wo_gemm_path(native.WO_DGRAD_W16, a, q, s, c, 300, 2**22, 8) == slow  # 256 rows of dy pass 2^31 bytes
+    assert lib.km_wo_gemm_path(native.WO_DGRAD_TRANSPOSED, a, q, s, c, 64, 256, 510) == tiled
+    assert lib.km_wo_gemm_path(native.WO_DGRAD_TRANSPOSED, a, q, s, c, 64, 2**22, 8) == slow
+    assert lib.km_wo_gemm_path(9, a, q, s, c, 1, 8, 8) < 0
+
+
 def test_wrappers_refuse_host_tensors():
     import pytest
     import torch

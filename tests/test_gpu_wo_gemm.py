@@ -203,6 +203,26 @@ def test_input_gradient_shapes_off_the_vector_path(fmt, recipe, m, n, k):
     assert_no_regression(dx.cpu(), eager, dy.double() @ w64, f"scalar dgrad {fmt} {recipe} {m}x{n}x{k}")
 
 
+def test_leaving_the_tiled_kernels_is_announced_once_per_shape():
+    """A ragged problem is served, correctly, by the one-thread-per-element kernel; the binding says so
+    once per direction and shape instead of leaving a silent cliff for the tuner to time."""
+    import warnings
+
+    x, q, scale, bias, dy = case(24, 40, 36, "int8", torch.bfloat16, seed=3)  # K % 8 != 0
+    native._SLOW_SEEN.clear()
+    with pytest.warns(native.SlowPathWarning, match="forward M=24 N=40 K=36"):
+        native.wo_gemm_fwd(x.cuda(), q.cuda(), scale.cuda(), None)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error", native.SlowPathWarning)
+        native.wo_gemm_fwd(x.cuda(), q.cuda(), scale.cuda(), None)  # the second call is silent
+        x2, q2, s2, _, dy2 = case(24, 64, 128, "int8", torch.bfloat16, seed=4)
+        native.wo_gemm_fwd(x2.cuda(), q2.cuda(), s2.cuda(), None)  # a shape the tiles take: no warning
+        native.wo_gemm_dgrad(dy2.cuda(), q2.cuda(), s2.cuda())
+    x3, q3, s3, _, dy3 = case(24, 36, 64, "int8", torch.bfloat16, seed=5)  # N % 8 != 0
+    with pytest.warns(native.SlowPathWarning, match="input gradient M=24 N=36 K=64"):
+        native.wo_gemm_dgrad(dy3.cuda(), q3.cuda(), s3.cuda())
+
+
 def test_int8_forward_is_exact_product_for_small_integers():
     """Integer activations and codes with unit scales: every product and partial sum is an
     integer below 2^24, so the kernel must reproduce the fp64 product exactly after the one
