@@ -32,3 +32,31 @@ def check_against_model(y16: torch.Tensor, ybf: torch.Tensor, model: np.ndarray,
         assert bool(((y.double() - want.double()).abs()[off] <= 1.0001 * unit[off]).all()), (what, dtype, "more than one unit from the rounded model")
         shares.append(share)
     return shares[1]
+
+
+def no_worse_than_eager(y: torch.Tensor, eager_y: torch.Tensor, truth: torch.Tensor, cut: float, what: str = "") -> dict:
+    """The reference's deep-K rule (mean abs / rel error no worse than the eager result's) with the one
+    allowance the instruction's summation needs: a result moved by `cut` (its mean distance from the exact
+    sum, measured against the instruction model) before its single rounding errs by at most `cut` more on
+    every element, that is by `cut` in abs_mean and by `cut * mean(1 / |truth|)` in rel_mean.
+
+    A mean of 1 / |truth| over everything is owned by the few outputs next to zero, and so is rel_mean
+    itself: both are taken over the outputs with |truth| >= 1 % of the median |truth| (the rest, a per cent
+    of a Gaussian output, is covered by abs_mean). The allowance must stay a small part of the eager
+    statistic it is added to, or the check would pass anything: asserted, and returned for the log."""
+    t = truth.detach().double().flatten()
+    keep = t.abs() >= 0.01 * t.abs().median()
+    assert keep.double().mean().item() > 0.95
+
+    def two(out):
+        err = (out.detach().double().flatten() - t).abs()
+        return err.mean().item(), (err[keep] / t[keep].abs()).mean().item()
+
+    eager_abs, eager_rel = two(eager_y)
+    got_abs, got_rel = two(y)
+    extra_abs, extra_rel = cut, cut * (1.0 / t[keep].abs()).mean().item()
+    assert extra_abs <= 0.25 * eager_abs and extra_rel <= 0.25 * eager_rel, (what, "the allowance swamps the statistic", extra_abs, eager_abs, extra_rel, eager_rel)
+    report = {"abs_mean": got_abs, "abs_allowed": eager_abs + extra_abs, "rel_mean": got_rel, "rel_allowed": eager_rel + extra_rel,
+              "abs_allowance_share": extra_abs / eager_abs, "rel_allowance_share": extra_rel / eager_rel}
+    assert got_abs <= eager_abs + extra_abs and got_rel <= eager_rel + extra_rel, (what, report)
+    return report
