@@ -8,6 +8,7 @@ _HOME = {
     "compute": ("ComputeCache", "ComputeWeight"),
     "convert": ("QuantLinear", "attach_compute", "default_filter", "quantize_model", "quantize_torch_linears"),
     "stored": ("attach_stored", "load_quantized", "quantized_state", "read_record", "save_quantized"),
+    "text": ("GroupQuantLinear", "linear_fate", "quantize_text_linears", "quantizes"),
     "weights": ("QuantWeight", "dequantize", "quantize"),
 }
 _WHERE = {name: module for module, names in _HOME.items() for name in names}

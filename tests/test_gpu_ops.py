@@ -164,6 +164,39 @@ def test_shortlist_is_timed_once_and_stored(tmp_path, monkeypatch):
     tuning._tables.clear()
 
 
+def test_text_encoder_linears_on_device():
+    """A text-encoder-shaped MLP of plain nn.Linear modules (4096 -> 12288 -> 4096 scaled down) quantized
+    in place on the card: weight-only int8 and fp8 through the weight-only kernels, mxfp8 through the
+    fp8 op, per-group int8 through its own module; outputs close to the dense ones, state keys under
+    `qweight`, and a kept fp32 linear fed 16-bit activations still runs."""
+    from kohakumosstrainer_amd.quant import GroupQuantLinear, QuantLinear, quantize_text_linears
+
+    def mlp():
+        torch.manual_seed(1)
+        m = nn.Sequential(nn.Linear(512, 1536), nn.GELU(), nn.Linear(1536, 512, bias=False)).to(DEV, torch.bfloat16)
+        return m
+
+    x = torch.randn(3, 50, 512, device=DEV, dtype=torch.bfloat16)
+    want = mlp()(x).float()
+    for precision, group, bound in (("int8", 0, 2e-2), ("fp8", 0, 6e-2), ("mxfp8", 0, 8e-2), ("int8", 128, 2e-2)):
+        m = mlp()
+        report = quantize_text_linears(m, precision, group, torch.bfloat16, recipe="mx")
+        assert report["layers"] == 2 and report["skipped"] == 0 and report["quant_bytes"] < report["dense_bytes"]
+        kind = GroupQuantLinear if group else QuantLinear
+        assert isinstance(m[0], kind) and isinstance(m[2], kind)
+        y = m(x)
+        assert y.dtype == torch.bfloat16 and y.shape == want.shape
+        rel = ((y.float() - want).norm() / want.norm()).item()
+        assert rel < bound, (precision, group, rel)
+        if not group:
+            assert any(k.startswith("0.qweight.") for k in m.state_dict())
+    from kohakumosstrainer_amd.model.linear import MossLinear as ML
+
+    kept = ML(512, 256).to(DEV)  # fp32 parameters, 16-bit activations
+    kept.init_weights(0.05)
+    assert kept(x).dtype == torch.bfloat16
+
+
 def test_modules_end_to_end_on_device():
     torch.manual_seed(0)
     model = nn.ModuleDict({"qkv": MossLinear(512, 1536, bias=True), "out": MossLinear(512, 512, bias=False)}).to(DEV, torch.bfloat16)
