@@ -35,14 +35,23 @@ constexpr int kBlkTileN = 128;
 // SA_KMAJOR: the activation scales are laid out [K/128, M] (the quantizer's second output), so
 // the 16 rows of an MFMA tile read one 64-byte run per step; from the natural [M, K/128] matrix
 // every lane gathers from a row of its own, which costs more than the MFMAs of the step.
-template <int OUT, int BM, int STAGES, bool SA_KMAJOR>
-__global__ __launch_bounds__(256) void gemm_fp8_blocks_kernel(
+// WAVES 8: two wavefronts per SIMD on the same tile (a 4 x 2 grid of (BM/4) x 64 sub-tiles). The loop
+// is scheduled by the compiler and its waits (slab and scale fetches, LDS reads, the promotion's
+// dependence on the MFMA) stand in the open with one wavefront per SIMD; a second one issues into them.
+// BN 256 (with WAVES 8): a 2 x 4 grid of 128 x 64 sub-tiles on a 256 x 256 tile, the operand bytes per
+// flop of the MX kernel's large tile; each half of the wavefronts has its own weight-scale block.
+template <int OUT, int BM, int STAGES, bool SA_KMAJOR, int WAVES = 4, int BN = kBlkTileN>
+__global__ __launch_bounds__(64 * WAVES) void gemm_fp8_blocks_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const float* __restrict__ sa,
     const float* __restrict__ sb, const uint16_t* __restrict__ bias, uint16_t* __restrict__ C, int M, int N, int K) {
-  constexpr int BN = kBlkTileN;
-  constexpr int TM = BM / 32, TN = BN / 32;     // 16x16 MFMA tiles per wavefront and axis
+  constexpr int WCOLS = BN / 64;                       // a wavefront's sub-tile is 64 columns wide
+  constexpr int NT = 64 * WAVES, WROWS = WAVES / WCOLS;  // wavefronts: WROWS along M x WCOLS along N
+  constexpr int TM = BM / (16 * WROWS), TN = 4;        // 16x16 MFMA tiles per wavefront and axis
+  static_assert(BN == 128 || (BN == 256 && WAVES == 8), "tile widths");
   constexpr int A_SLAB = BM * kStepBytes, B_SLAB = BN * kStepBytes;
-  constexpr int A_PASSES = BM / 32, B_PASSES = BN / 32;  // 32 rows (4 KiB) per pass of 256 lanes
+  constexpr int PASS_ROWS = NT / 8, PASS_BYTES = NT * 16;  // 8 lanes per 128-byte row
+  constexpr int A_PASSES = BM / PASS_ROWS, B_PASSES = BN / PASS_ROWS;
+  static_assert(WAVES == 4 || WAVES == 8, "one or two wavefronts per SIMD");
   constexpr int DMAS = A_PASSES + B_PASSES;     // slab fetch instructions per wavefront and step
   static_assert(STAGES == 2 || STAGES == 3, "ring of two or three slab pairs");
   static_assert(STAGES * (A_SLAB + B_SLAB) <= 160 * 1024, "LDS");
@@ -55,7 +64,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_blocks_kernel(
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
+  // wavefront index bits: column within a 128-column half, row, (BN 256) which half
+  const int wm = (BN == 256 ? (wave >> 1) & 1 : wave >> 1) * (BM / WROWS), wn = (BN == 256 ? (wave >> 2) * 128 : 0) + (wave & 1) * 64;
   const int r16 = lane & 15, g = lane >> 4;
   const int nk = K / kStepBytes;
 
@@ -67,13 +77,13 @@ __global__ __launch_bounds__(256) void gemm_fp8_blocks_kernel(
   const int srow = ((w >> 4) << 4) + ((w & 1) << 3) + ((w >> 1) & 7);
   const int src_chunk = (tid & 7) ^ (srow & 7);
   const int ld_voff = srow * K + src_chunk * 16;
-  const int pass_stride = 32 * K;
+  const int pass_stride = PASS_ROWS * K;
   auto dma = [&](uint8_t* abuf, uint8_t* bbuf, int ks) __attribute__((always_inline)) {
     const int koff = __builtin_amdgcn_readfirstlane(ks * kStepBytes);
 #pragma unroll
-    for (int i = 0; i < A_PASSES; ++i) hidden_dma_b128(a_rsrc, lds_offset(abuf) + i * 4096 + wave * 1024, ld_voff + i * pass_stride, koff);
+    for (int i = 0; i < A_PASSES; ++i) hidden_dma_b128(a_rsrc, lds_offset(abuf) + i * PASS_BYTES + wave * 1024, ld_voff + i * pass_stride, koff);
 #pragma unroll
-    for (int i = 0; i < B_PASSES; ++i) hidden_dma_b128(b_rsrc, lds_offset(bbuf) + i * 4096 + wave * 1024, ld_voff + i * pass_stride, koff);
+    for (int i = 0; i < B_PASSES; ++i) hidden_dma_b128(b_rsrc, lds_offset(bbuf) + i * PASS_BYTES + wave * 1024, ld_voff + i * pass_stride, koff);
   };
   auto fragment = [&](const uint8_t* slab, int row) __attribute__((always_inline)) -> v8i {
     const v4i lo = *reinterpret_cast<const v4i*>(slab + slab_offset(row, g));
@@ -93,7 +103,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_blocks_kernel(
   const v4i sa_rsrc = SA_KMAJOR ? raw_rsrc(sa, (uint32_t)min((int64_t)M * nk * 4, (int64_t)0x7FFFFFFF))
                                 : raw_rsrc(sa + (size_t)m0 * nk, (uint32_t)min((int64_t)(M - m0) * nk * 4, (int64_t)0x7FFFFFFF));
   const int sa_voff = SA_KMAJOR ? (m0 + wm + r16) * 4 : (wm + r16) * nk * 4;
-  const float* sb_row = sb + (size_t)tile_n * nk;
+  const float* sb_row = sb + (size_t)min((n0 + wn) >> 7, (N - 1) >> 7) * nk;  // the wavefront's 128-column weight block
   uint32_t sa_raw[TM];
   auto sa_fetch = [&](int ks) __attribute__((always_inline)) {
 #pragma unroll
@@ -192,33 +202,46 @@ __global__ __launch_bounds__(256) void gemm_fp8_blocks_kernel(
   // every fetch has landed and every wavefront is past its last LDS read: the ring is free
   uint8_t* ea = &a_ring[0][0];
   uint8_t* eb = &b_ring[0][0];
-  store_tile<BM, BN, OUT, 0, false, false>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, m0, n0, ea, ea + 16384, eb, eb + 16384);
+  if constexpr (WAVES == 4) {
+    store_tile<BM, BN, OUT, 0, false, false>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, m0, n0, ea, ea + 16384, eb, eb + 16384);
+  } else if constexpr (BN == 128) {
+    // each group of four wavefronts writes its half of the tile's rows, staging in a ring of its own
+    uint8_t* stage = wave < 4 ? ea : eb;
+    store_tile<BM / 2, BN, OUT, 0, false, false>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, m0 + (wave >> 2) * (BM / 2), n0, stage, stage + 4096,
+                                                 stage + 8192, stage + 12288);
+  } else {
+    // each group of four wavefronts writes its 128-column half of the tile
+    uint8_t* stage = wave < 4 ? ea : eb;
+    store_tile<BM, 128, OUT, 0, false, false>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, m0, n0 + (wave >> 2) * 128, stage, stage + 4096,
+                                              stage + 8192, stage + 12288);
+  }
 }
 
 struct BlocksConfig {
-  int bm, stages;
+  int bm, stages, waves, bn;
 };
-// the tall tile first (fewest operand and LDS bytes per flop); the square one for short M and small grids
-static const BlocksConfig kBlocksConfigs[] = {{256, 3}, {128, 2}};
-constexpr int kNumBlocksConfigs = 2;
+// the tall tile first (fewest operand and LDS bytes per flop); the square one for short M and small grids;
+// the tall tile with two wavefronts per SIMD
+static const BlocksConfig kBlocksConfigs[] = {{256, 3, 4, 128}, {128, 2, 4, 128}, {256, 3, 8, 128}, {256, 2, 8, 256}};
+constexpr int kNumBlocksConfigs = 4;
 
 int blocks_gemm_num_configs() { return kNumBlocksConfigs; }
 int blocks_gemm_config_desc(int config, char* buf, int len) {
   if (config < 0 || config >= kNumBlocksConfigs) return km_fail(KM_ERR_ARG, "config out of range");
   const BlocksConfig& c = kBlocksConfigs[config];
-  snprintf(buf, len, "bm=%d,bn=%d,bk=128,waves=4,stages=%d,wg_per_cu=%d", c.bm, kBlkTileN, c.stages, c.bm == 256 ? 1 : 2);
+  snprintf(buf, len, "bm=%d,bn=%d,bk=128,waves=%d,stages=%d,wg_per_cu=%d", c.bm, c.bn, c.waves, c.stages, c.bm == 256 ? 1 : 2);
   return KM_OK;
 }
 
-template <int OUT, int BM, int STAGES>
+template <int OUT, int BM, int STAGES, int WAVES = 4, int BN = kBlkTileN>
 static void launch_blocks(const void* a, const float* sa, const void* b, const float* sb, const void* bias, void* c,
                           int M, int N, int K, bool sa_kmajor, hipStream_t st) {
-  const int tiles = ((M + BM - 1) / BM) * ((N + kBlkTileN - 1) / kBlkTileN);
+  const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   if (sa_kmajor)
-    hipLaunchKernelGGL((gemm_fp8_blocks_kernel<OUT, BM, STAGES, true>), dim3(tiles), dim3(256), 0, st, (const uint8_t*)a,
+    hipLaunchKernelGGL((gemm_fp8_blocks_kernel<OUT, BM, STAGES, true, WAVES, BN>), dim3(tiles), dim3(64 * WAVES), 0, st, (const uint8_t*)a,
                        (const uint8_t*)b, sa, sb, (const uint16_t*)bias, (uint16_t*)c, M, N, K);
   else
-    hipLaunchKernelGGL((gemm_fp8_blocks_kernel<OUT, BM, STAGES, false>), dim3(tiles), dim3(256), 0, st, (const uint8_t*)a,
+    hipLaunchKernelGGL((gemm_fp8_blocks_kernel<OUT, BM, STAGES, false, WAVES, BN>), dim3(tiles), dim3(64 * WAVES), 0, st, (const uint8_t*)a,
                        (const uint8_t*)b, sa, sb, (const uint16_t*)bias, (uint16_t*)c, M, N, K);
 }
 
@@ -243,10 +266,14 @@ extern "C" int km_gemm_fp8_blocks(const void* a, const float* sa, const void* b,
   const bool km = sa_layout == KM_SCALES_KMAJOR;
   if (out_dtype == KM_BF16) {
     if (config == 0) launch_blocks<KM_BF16, 256, 3>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
-    else launch_blocks<KM_BF16, 128, 2>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
+    else if (config == 1) launch_blocks<KM_BF16, 128, 2>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
+    else if (config == 2) launch_blocks<KM_BF16, 256, 3, 8>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
+    else launch_blocks<KM_BF16, 256, 2, 8, 256>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
   } else {
     if (config == 0) launch_blocks<KM_F16, 256, 3>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
-    else launch_blocks<KM_F16, 128, 2>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
+    else if (config == 1) launch_blocks<KM_F16, 128, 2>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
+    else if (config == 2) launch_blocks<KM_F16, 256, 3, 8>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
+    else launch_blocks<KM_F16, 256, 2, 8, 256>(a, sa, b, sb, bias, c, (int)M, (int)N, (int)K, km, st);
   }
   return km_check_launch("km_gemm_fp8_blocks");
 }

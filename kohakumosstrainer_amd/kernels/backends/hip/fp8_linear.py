@@ -43,9 +43,11 @@ def candidates(recipe: str, m: int, n: int | None = None, k: int | None = None) 
     fits = [c for c in cfgs if c["bm"] <= limit] or cfgs
     ranked = sorted(fits, key=lambda c: -(c["bm"] * c["bn"]) if m >= 1024 else c["bm"])
     if recipe == "block":
-        # measured at M16384 K3072 N9216: the 128 x 128 tile (two workgroups per compute unit) 0.48 ms,
-        # the 256 x 128 tile 0.55 ms
-        ranked = sorted(fits, key=lambda c: c["bm"])
+        # measured at M16384 K3072 N9216: the 256 x 256 tile with two wavefronts per SIMD 0.42 ms, the
+        # 128 x 128 tile (two workgroups per compute unit) 0.47 ms, the 256 x 128 tile 0.50 ms with eight
+        # wavefronts and 0.54 ms with four. Short M and narrow N keep the small tile first.
+        big = m >= 1024 and (n is None or n >= 512)
+        ranked = sorted(fits, key=lambda c: (not (big and c["bn"] == 256), c["bm"], -c.get("waves", 4)))
     if recipe in ("mx", "row", "block") and m <= native.FUSED_MAX_M and (n is None or n % 32 == 0) and (k is None or k % 128 == 0):
         # measured at K3072 N9216, one launch against quantizer + GEMM. mx: 9.1 against 19 us at M = 1,
         # 11.0 against 21 at M = 16, 15.4 against 21 at M = 32 (even at 48); block: 10.6 against 21.4, 12.2
