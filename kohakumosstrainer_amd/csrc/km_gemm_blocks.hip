@@ -23,6 +23,8 @@
 // matrix pipe, bounds 64 x 64 sub-tiles).
 #include <stdio.h>
 
+#include <mutex>
+
 #include "km_gemm_common.h"
 
 namespace km {
@@ -33,8 +35,8 @@ constexpr int kBlkTileN = 128;
 // the compiler puts their results in accumulation registers and copies every partial sum out
 // before the promotion (one more vector-ALU instruction per value).
 // SA_KMAJOR: the activation scales are laid out [K/128, M] (the quantizer's second output), so
-// the 16 rows of an MFMA tile read one 64-byte run per step; from the natural [M, K/128] matrix
-// every lane gathers from a row of its own, which costs more than the MFMAs of the step.
+// the tile's scales of a step are one run of BM floats; from the natural [M, K/128] matrix every
+// lane of the scale fetch gathers from a row of its own.
 // WAVES 8: two wavefronts per SIMD on the same tile (a 4 x 2 grid of (BM/4) x 64 sub-tiles). The loop
 // is scheduled by the compiler and its waits (slab and scale fetches, LDS reads, the promotion's
 // dependence on the MFMA) stand in the open with one wavefront per SIMD; a second one issues into them.
@@ -58,10 +60,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fp8_blocks_kernel(
   static_assert(STAGES * A_SLAB >= 2 * 16384 && STAGES * B_SLAB >= 2 * 16384, "epilogue staging: four 16 KiB buffers");
   __shared__ __attribute__((aligned(1024))) uint8_t a_ring[STAGES][A_SLAB];
   __shared__ __attribute__((aligned(1024))) uint8_t b_ring[STAGES][B_SLAB];
+  __shared__ __attribute__((aligned(256))) float sa_ring[STAGES][BM];  // the tile's activation scales of a step
 
-  int tile_m, tile_n;
-  tile_of(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, tile_n);
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // wavefront index bits: column within a 128-column half, row, (BN 256) which half
@@ -69,21 +69,63 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fp8_blocks_kernel(
   const int r16 = lane & 15, g = lane >> 4;
   const int nk = K / kStepBytes;
 
-  // rows past the end are fetched as zeros by the descriptors' range check
-  const v4i a_rsrc = raw_rsrc(A + (size_t)m0 * K, (uint32_t)min((int64_t)(M - m0) * K, (int64_t)0x7FFFFFFF));
-  const v4i b_rsrc = raw_rsrc(B + (size_t)n0 * K, (uint32_t)min((int64_t)(N - n0) * K, (int64_t)0x7FFFFFFF));
+  // What a tile fixes: its corner, the operand descriptors (rows past the end are fetched as zeros by
+  // their range check), the activation-scale descriptor and lane offset, the wavefront's weight-scale row.
+  //
+  // Activation scales of a step: the tile's BM floats go to LDS with BM / 64 fetches of 4 bytes per lane
+  // (one each by the first wavefronts), like the slabs from inline asm: a load the compiler sees would
+  // make it wait for every fetch in flight where the value is first used (its count does not include the
+  // hidden ones). A lane needs the scales of rows j * 16 + r16 (j < TM) of its wavefront's 16 * TM rows,
+  // so the fetch scatters: LDS float i of the ring slot holds row (i / (16 TM)) * 16 TM + (i % TM) * 16 +
+  // (i / TM) % 16, and a lane reads its TM scales as one or two 16-byte LDS reads. (One 4-byte global load
+  // per scale and lane, TM a step and wavefront, held the matrix pipe up for a sixth of the kernel's time.)
+  // Natural layout: the descriptor starts at the tile's first row, so rows past M read as zero scales
+  // (their partial sums are zeros as well). K-major: a row past M reads a neighbour's scale or, past the
+  // end, zero; its sums are never stored.
+  struct Tile {
+    int m0, n0, sa_voff;
+    v4i a_rsrc, b_rsrc, sa_rsrc;
+    const float* sb_row;
+  };
+  constexpr int SA_FETCHES = BM / 64;  // wavefront w < SA_FETCHES fetches LDS floats [64 w, 64 w + 64) of a slot
+  static_assert(SA_FETCHES <= WAVES, "one scale fetch per wavefront at most");
+  const int sa_slot_index = (wave * 64 + lane) % BM;
+  const int sa_row = sa_slot_index / (16 * TM) * (16 * TM) + (sa_slot_index % TM) * 16 + (sa_slot_index / TM) % 16;
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  auto tile_at = [&](int pid) __attribute__((always_inline)) -> Tile {
+    int tile_m, tile_n;
+    tile_of(pid, tiles_m, tiles_n, tile_m, tile_n);
+    Tile t;
+    t.m0 = tile_m * BM;
+    t.n0 = tile_n * BN;
+    t.a_rsrc = raw_rsrc(A + (size_t)t.m0 * K, (uint32_t)min((int64_t)(M - t.m0) * K, (int64_t)0x7FFFFFFF));
+    t.b_rsrc = raw_rsrc(B + (size_t)t.n0 * K, (uint32_t)min((int64_t)(N - t.n0) * K, (int64_t)0x7FFFFFFF));
+    t.sa_rsrc = SA_KMAJOR ? raw_rsrc(sa, (uint32_t)min((int64_t)M * nk * 4, (int64_t)0x7FFFFFFF))
+                          : raw_rsrc(sa + (size_t)t.m0 * nk, (uint32_t)min((int64_t)(M - t.m0) * nk * 4, (int64_t)0x7FFFFFFF));
+    t.sa_voff = SA_KMAJOR ? (t.m0 + sa_row) * 4 : sa_row * nk * 4;
+    t.sb_row = sb + (size_t)min((t.n0 + wn) >> 7, (N - 1) >> 7) * nk;  // the wavefront's 128-column weight block
+    return t;
+  };
+  // PERSIST: a work-group walks tiles pid, pid + grid, ... and fetches the first slabs and scales of
+  // the tile after this one during this tile's last K step, so only the epilogue stands between the
+  // MFMAs of two tiles. The epilogue stages in the slot the last step read, the early slabs land in the
+  // other one, which the walk takes for slot 0 again: the host launches fewer work-groups than tiles
+  // only when the number of K steps is even.
+  constexpr bool PERSIST = WAVES == 8 && STAGES == 2;
+  int pid = blockIdx.x;
+  Tile T = tile_at(pid);
   // staging map of a pass: 8 lanes per row; 16 lanes cover rows r and r+8 (one LDS line)
   const int w = tid >> 3;
   const int srow = ((w >> 4) << 4) + ((w & 1) << 3) + ((w >> 1) & 7);
   const int src_chunk = (tid & 7) ^ (srow & 7);
   const int ld_voff = srow * K + src_chunk * 16;
   const int pass_stride = PASS_ROWS * K;
-  auto dma = [&](uint8_t* abuf, uint8_t* bbuf, int ks) __attribute__((always_inline)) {
+  auto dma = [&](const Tile& t, uint8_t* abuf, uint8_t* bbuf, int ks) __attribute__((always_inline)) {
     const int koff = __builtin_amdgcn_readfirstlane(ks * kStepBytes);
 #pragma unroll
-    for (int i = 0; i < A_PASSES; ++i) hidden_dma_b128(a_rsrc, lds_offset(abuf) + i * PASS_BYTES + wave * 1024, ld_voff + i * pass_stride, koff);
+    for (int i = 0; i < A_PASSES; ++i) hidden_dma_b128(t.a_rsrc, lds_offset(abuf) + i * PASS_BYTES + wave * 1024, ld_voff + i * pass_stride, koff);
 #pragma unroll
-    for (int i = 0; i < B_PASSES; ++i) hidden_dma_b128(b_rsrc, lds_offset(bbuf) + i * PASS_BYTES + wave * 1024, ld_voff + i * pass_stride, koff);
+    for (int i = 0; i < B_PASSES; ++i) hidden_dma_b128(t.b_rsrc, lds_offset(bbuf) + i * PASS_BYTES + wave * 1024, ld_voff + i * pass_stride, koff);
   };
   auto fragment = [&](const uint8_t* slab, int row) __attribute__((always_inline)) -> v8i {
     const v4i lo = *reinterpret_cast<const v4i*>(slab + slab_offset(row, g));
@@ -91,129 +133,138 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fp8_blocks_kernel(
     return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
 
-  // Scales of this lane's TM token rows and of the tile's weight block.
-  // The activation scales are fetched like the slabs, from inline asm: a load the compiler sees
-  // would make it wait for every fetch in flight (its count does not include the hidden ones)
-  // where the value is first used. The fetched registers are read once, by an opaque move placed
-  // right after the step's own wait.
-  // The descriptor starts at this tile's first row: rows past M read as zero scales (their
-  // partial sums are zeros as well). Row j * 16 + r16 of the sub-tile: the lane part of the
-  // offset is one register, the row-group part is uniform.
-  // (K-major: a row past M reads a neighbour's scale or, past the end, zero; its sums are never stored.)
-  const v4i sa_rsrc = SA_KMAJOR ? raw_rsrc(sa, (uint32_t)min((int64_t)M * nk * 4, (int64_t)0x7FFFFFFF))
-                                : raw_rsrc(sa + (size_t)m0 * nk, (uint32_t)min((int64_t)(M - m0) * nk * 4, (int64_t)0x7FFFFFFF));
-  const int sa_voff = SA_KMAJOR ? (m0 + wm + r16) * 4 : (wm + r16) * nk * 4;
-  const float* sb_row = sb + (size_t)min((n0 + wn) >> 7, (N - 1) >> 7) * nk;  // the wavefront's 128-column weight block
-  uint32_t sa_raw[TM];
-  auto sa_fetch = [&](int ks) __attribute__((always_inline)) {
-#pragma unroll
-    for (int j = 0; j < TM; ++j)
-      sa_raw[j] = hidden_load_b32(sa_rsrc, sa_voff, __builtin_amdgcn_readfirstlane(SA_KMAJOR ? (ks * M + j * 16) * 4 : (ks + j * 16 * nk) * 4));
+  // the activation scales of step ks of tile t, into ring slot `slot`
+  auto sa_fetch = [&](const Tile& t, int ks, int slot) __attribute__((always_inline)) {
+    if (wave < SA_FETCHES)
+      hidden_touch_b32(t.sa_rsrc, lds_offset(&sa_ring[slot][0]) + wave * 256, t.sa_voff, __builtin_amdgcn_readfirstlane(SA_KMAJOR ? ks * M * 4 : ks * 4));
   };
-  float sa_next[TM];
-  auto sa_take = [&]() __attribute__((always_inline)) {
-#pragma unroll
-    for (int j = 0; j < TM; ++j) asm volatile("v_mov_b32 %0, %1" : "=v"(sa_next[j]) : "v"(sa_raw[j]));
-  };
+  const int sa_lane = wm + r16 * TM;  // first of this lane's TM floats in a slot
 
-  v4f acc[TN][TM];
-#pragma unroll
-  for (int t = 0; t < TN; ++t)
-#pragma unroll
-    for (int j = 0; j < TM; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
-
-  // raw scales of the step ahead: fetched a step early, multiplied once that step begins
-  float sb_next = sb_row[0];
+  // weight scale of the step ahead: fetched a step early
+  float sb_next = T.sb_row[0];
   // prologue: the scales of step 0 and the slabs of the first STAGES - 1 steps; wait for step 0 only
-  sa_fetch(0);
-  dma(a_ring[0], b_ring[0], 0);
+  sa_fetch(T, 0, 0);
+  dma(T, a_ring[0], b_ring[0], 0);
   if (STAGES == 3 && nk > 1) {
-    dma(a_ring[1], b_ring[1], 1);
+    dma(T, a_ring[1], b_ring[1], 1);
     __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(DMAS));
   } else {
     __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
   }
   __syncthreads();
   __builtin_amdgcn_sched_barrier(0);
-  sa_take();
 
-  // One K step: the slabs of step ks are in ring slot `cur`; slot `pre` (read last in the step
-  // before, behind that step's barrier) takes the slabs of step ks + STAGES - 1.
-  auto step = [&](int ks, auto cur_tag, auto pre_tag) __attribute__((always_inline)) {
-    constexpr int cur = decltype(cur_tag)::value, pre = decltype(pre_tag)::value;
-    const uint8_t* a_cur = a_ring[cur];
-    const uint8_t* b_cur = b_ring[cur];
-    float s_cur[TM];
+  const int total = tiles_m * tiles_n;
+  for (;;) {
+    const int pid_after = pid + (int)gridDim.x;
+    const bool more = PERSIST && pid_after < total;
+    const Tile U = tile_at(more ? pid_after : pid);  // the tile after this one
+
+    v4f acc[TN][TM];
 #pragma unroll
-    for (int j = 0; j < TM; ++j) s_cur[j] = sa_next[j] * sb_next;
-    sb_next = sb_row[min(ks + 1, nk - 1)];
-    sa_fetch(min(ks + 1, nk - 1));
-    const bool ahead = ks + STAGES - 1 < nk;
-    if (ahead) dma(a_ring[pre], b_ring[pre], ks + STAGES - 1);
-    v8i wf[TN];
+    for (int t = 0; t < TN; ++t)
 #pragma unroll
-    for (int t = 0; t < TN; ++t) wf[t] = fragment(b_cur, wn + t * 16 + r16);
-    v8i xf = fragment(a_cur, wm + r16);
-    v4f part[2][TN];
-    static_for<TM + 1>([&](auto j_tag) __attribute__((always_inline)) {
-      constexpr int j = decltype(j_tag)::value;
-      v8i xf_next = xf;
-      if constexpr (j + 1 < TM) xf_next = fragment(a_cur, wm + (j + 1) * 16 + r16);
-      static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
-        constexpr int t = decltype(t_tag)::value;
-        // MFMA rows come from B (output columns n), MFMA columns from A (tokens m); unit scales
-        if constexpr (j < TM)
-          part[j & 1][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[t], xf, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
-        if constexpr (j > 0) {
+      for (int j = 0; j < TM; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    // One K step: the slabs of step ks are in ring slot `cur`; slot `pre` (read last in the step
+    // before, behind that step's barrier) takes the slabs of step ks + STAGES - 1 or, in the last step
+    // of a tile that has a successor, the successor's first.
+    auto step = [&](int ks, auto cur_tag, auto pre_tag) __attribute__((always_inline)) {
+      constexpr int cur = decltype(cur_tag)::value, pre = decltype(pre_tag)::value;
+      const uint8_t* a_cur = a_ring[cur];
+      const uint8_t* b_cur = b_ring[cur];
+      constexpr int nxt = (cur + 1) % STAGES;  // ring slot of step ks + 1
+      float s_cur[TM];
 #pragma unroll
-          for (int v = 0; v < 4; ++v) acc[t][j - 1][v] = __builtin_fmaf(part[(j - 1) & 1][t][v], s_cur[j - 1], acc[t][j - 1][v]);
-          // pins the promotion ahead of the wait below (the compiler would sink it past the barrier)
-          asm volatile("" : "+v"(acc[t][j - 1]));
-        }
-        __builtin_amdgcn_sched_barrier(0);
+      for (int j4 = 0; j4 < TM; j4 += 4) {
+        const v4f four = *reinterpret_cast<const v4f*>(&sa_ring[cur][sa_lane + j4]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s_cur[j4 + j] = four[j] * sb_next;
+      }
+      const bool ahead = ks + STAGES - 1 < nk;
+      if (more && ks == nk - 1) {
+        sb_next = U.sb_row[0];
+        sa_fetch(U, 0, nxt);
+        dma(U, a_ring[pre], b_ring[pre], 0);
+      } else {
+        sb_next = T.sb_row[min(ks + 1, nk - 1)];
+        sa_fetch(T, min(ks + 1, nk - 1), nxt);
+        if (ahead) dma(T, a_ring[pre], b_ring[pre], ks + STAGES - 1);
+      }
+      v8i wf[TN];
+#pragma unroll
+      for (int t = 0; t < TN; ++t) wf[t] = fragment(b_cur, wn + t * 16 + r16);
+      v8i xf = fragment(a_cur, wm + r16);
+      v4f part[2][TN];
+      static_for<TM + 1>([&](auto j_tag) __attribute__((always_inline)) {
+        constexpr int j = decltype(j_tag)::value;
+        v8i xf_next = xf;
+        if constexpr (j + 1 < TM) xf_next = fragment(a_cur, wm + (j + 1) * 16 + r16);
+        static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
+          constexpr int t = decltype(t_tag)::value;
+          // MFMA rows come from B (output columns n), MFMA columns from A (tokens m); unit scales
+          if constexpr (j < TM)
+            part[j & 1][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[t], xf, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+          if constexpr (j > 0) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[t][j - 1][v] = __builtin_fmaf(part[(j - 1) & 1][t][v], s_cur[j - 1], acc[t][j - 1][v]);
+            // pins the promotion ahead of the wait below (the compiler would sink it past the barrier)
+            asm volatile("" : "+v"(acc[t][j - 1]));
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        });
+        xf = xf_next;
       });
-      xf = xf_next;
-    });
-    // The slabs and scales of step ks + 1 must have landed (STAGES 3: the DMAS newest fetches, those
-    // of step ks + 2, stay in flight: vector-memory results return in order) and this step's LDS reads
-    // must be done before the barrier lets another wavefront overwrite the slot.
-    if (STAGES == 3 && ahead) __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(DMAS));
-    else __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
-    __syncthreads();
-    __builtin_amdgcn_sched_barrier(0);
-    sa_take();
-  };
-  using i0 = std::integral_constant<int, 0>;
-  using i1 = std::integral_constant<int, 1>;
-  using i2 = std::integral_constant<int, 2>;
-  if constexpr (STAGES == 2) {
-    for (int ks = 0; ks < nk; ks += 2) {
-      step(ks, i0{}, i1{});
-      if (ks + 1 < nk) step(ks + 1, i1{}, i0{});
+      // The slabs and scales of step ks + 1 must have landed (STAGES 3: the DMAS newest fetches, those
+      // of step ks + 2, stay in flight: vector-memory results return in order) and this step's LDS reads
+      // must be done before the barrier lets another wavefront overwrite the slot.
+      if (STAGES == 3 && ahead) __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(DMAS));
+      else __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    using i0 = std::integral_constant<int, 0>;
+    using i1 = std::integral_constant<int, 1>;
+    using i2 = std::integral_constant<int, 2>;
+    if constexpr (STAGES == 2) {
+      for (int ks = 0; ks < nk; ks += 2) {
+        step(ks, i0{}, i1{});
+        if (ks + 1 < nk) step(ks + 1, i1{}, i0{});
+      }
+    } else {
+      for (int ks = 0; ks < nk; ks += 3) {
+        step(ks, i0{}, i2{});
+        if (ks + 1 < nk) step(ks + 1, i1{}, i0{});
+        if (ks + 2 < nk) step(ks + 2, i2{}, i1{});
+      }
     }
-  } else {
-    for (int ks = 0; ks < nk; ks += 3) {
-      step(ks, i0{}, i2{});
-      if (ks + 1 < nk) step(ks + 1, i1{}, i0{});
-      if (ks + 2 < nk) step(ks + 2, i2{}, i1{});
-    }
-  }
 
-  // every fetch has landed and every wavefront is past its last LDS read: the ring is free
-  uint8_t* ea = &a_ring[0][0];
-  uint8_t* eb = &b_ring[0][0];
-  if constexpr (WAVES == 4) {
-    store_tile<BM, BN, OUT, 0, false, false>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, m0, n0, ea, ea + 16384, eb, eb + 16384);
-  } else if constexpr (BN == 128) {
-    // each group of four wavefronts writes its half of the tile's rows, staging in a ring of its own
-    uint8_t* stage = wave < 4 ? ea : eb;
-    store_tile<BM / 2, BN, OUT, 0, false, false>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, m0 + (wave >> 2) * (BM / 2), n0, stage, stage + 4096,
-                                                 stage + 8192, stage + 12288);
-  } else {
-    // each group of four wavefronts writes its 128-column half of the tile
-    uint8_t* stage = wave < 4 ? ea : eb;
-    store_tile<BM, 128, OUT, 0, false, false>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, m0, n0 + (wave >> 2) * 128, stage, stage + 4096,
-                                              stage + 8192, stage + 12288);
+    // Every fetch has landed and every wavefront is past its last LDS read. The slot of the last step
+    // is free for staging (with a successor, the other slot holds its first slabs).
+    const int last_slot = (nk - 1) % STAGES;
+    uint8_t* ea = &a_ring[0][0] + last_slot * A_SLAB;
+    uint8_t* eb = &b_ring[0][0] + last_slot * B_SLAB;
+    if constexpr (WAVES == 4) {
+      // four 16 KiB buffers: with the square tile they are the whole ring
+      ea = &a_ring[0][0];
+      eb = &b_ring[0][0];
+      store_tile<BM, BN, OUT, 0, false, false>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, T.m0, T.n0, ea, ea + 16384, eb, eb + 16384);
+    } else if constexpr (BN == 128) {
+      // each group of four wavefronts writes its half of the tile's rows, staging in a ring of its own
+      uint8_t* stage = wave < 4 ? ea : eb;
+      store_tile<BM / 2, BN, OUT, 0, false, false>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, T.m0 + (wave >> 2) * (BM / 2), T.n0, stage, stage + 4096,
+                                                   stage + 8192, stage + 12288);
+    } else {
+      // each group of four wavefronts writes its 128-column half of the tile
+      uint8_t* stage = wave < 4 ? ea : eb;
+      store_tile<BM, 128, OUT, 0, false, false>(acc, 1.0f, nullptr, nullptr, bias, C, M, N, T.m0, T.n0 + (wave >> 2) * 128, stage, stage + 4096,
+                                                stage + 8192, stage + 12288);
+    }
+    if (!more) break;
+    // the staging reads are done before the successor's step 0 fetches into this slot
+    __syncthreads();
+    pid = pid_after;
+    T = U;
   }
 }
 
@@ -233,15 +284,38 @@ int blocks_gemm_config_desc(int config, char* buf, int len) {
   return KM_OK;
 }
 
+// compute units of the current device, asked once per device
+static int compute_units() {
+  static std::mutex mu;
+  static int seen[64];
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 0;
+  std::lock_guard<std::mutex> lock(mu);
+  if (seen[device] == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
+    seen[device] = cus;
+  }
+  return seen[device];
+}
+
 template <int OUT, int BM, int STAGES, int WAVES = 4, int BN = kBlkTileN>
 static void launch_blocks(const void* a, const float* sa, const void* b, const float* sb, const void* bias, void* c,
                           int M, int N, int K, bool sa_kmajor, hipStream_t st) {
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  // The kernel that walks tiles (two stages, eight wavefronts) holds one work-group per compute unit:
+  // launch one per unit, a multiple of the 8 XCDs so that tile pid + grid stays on the XCD of tile pid.
+  // An odd number of K steps would leave the early slabs in the wrong ring slot: one work-group per tile then.
+  int grid = tiles;
+  if (WAVES == 8 && STAGES == 2 && (K / kStepBytes) % 2 == 0) {
+    const int units = compute_units();
+    if (units >= kXcds && units - units % kXcds < tiles) grid = units - units % kXcds;
+  }
   if (sa_kmajor)
-    hipLaunchKernelGGL((gemm_fp8_blocks_kernel<OUT, BM, STAGES, true, WAVES, BN>), dim3(tiles), dim3(64 * WAVES), 0, st, (const uint8_t*)a,
+    hipLaunchKernelGGL((gemm_fp8_blocks_kernel<OUT, BM, STAGES, true, WAVES, BN>), dim3(grid), dim3(64 * WAVES), 0, st, (const uint8_t*)a,
                        (const uint8_t*)b, sa, sb, (const uint16_t*)bias, (uint16_t*)c, M, N, K);
   else
-    hipLaunchKernelGGL((gemm_fp8_blocks_kernel<OUT, BM, STAGES, false, WAVES, BN>), dim3(tiles), dim3(64 * WAVES), 0, st, (const uint8_t*)a,
+    hipLaunchKernelGGL((gemm_fp8_blocks_kernel<OUT, BM, STAGES, false, WAVES, BN>), dim3(grid), dim3(64 * WAVES), 0, st, (const uint8_t*)a,
                        (const uint8_t*)b, sa, sb, (const uint16_t*)bias, (uint16_t*)c, M, N, K);
 }
 
