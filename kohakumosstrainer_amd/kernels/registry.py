@@ -206,9 +206,16 @@ def _records_grad(args) -> bool:
     return (
         torch.is_grad_enabled()
         and not torch.compiler.is_compiling()
-        and torch._C._autograd._top_saved_tensors_default_hooks(False) is None
+        and not _saved_tensor_hooks_active()
         and any(isinstance(a, torch.Tensor) and a.requires_grad for a in args)
     )
+
+
+def _saved_tensor_hooks_active() -> bool:
+    probe = getattr(torch._C._autograd, "_top_saved_tensors_default_hooks", None)
+    if probe is None:
+        return True  # cannot tell: leave such a call unguarded rather than change what its hooks see
+    return probe(False) is not None
 
 
 def _as_leaves(args) -> list:
@@ -248,7 +255,8 @@ class _Guarded(torch.autograd.Function):
         try:
             try:
                 got = _backprop(ctx.outs, ctx.leaves, grads)
-                _S.proven.add(bound)
+                with _S.lock:  # backward runs on autograd's threads
+                    _S.proven.add(bound)
             except LAUNCH_ERRORS as err:
                 saved = iter(ctx.saved_tensors)
                 args = [next(saved) if slot is None else slot[0] for slot in ctx.others]
@@ -330,7 +338,7 @@ class Bound:
     def fall_back(self, err: BaseException, args=None, kwargs=None) -> None:
         """Leave the current backend after `err`. Returns with the op (and its siblings) bound to
         the next usable backend, or raises: `err` itself when it must not be answered by moving on,
-        `InputError` when the arguments are at fault, `NoImplementationError`-free `err` when the chain ends."""
+        `InputError` when the arguments are at fault, `err` again when no backend is left in the chain."""
         if self.pinned or not is_build_error(err) or is_sticky_error(err, self.device):
             raise err
         if not isinstance(err, BackendUnavailable) and args is not None:
