@@ -196,33 +196,34 @@ def test_block_gemm_against_fp64(dtype, m, n, k):
         first = y
 
 
-@pytest.mark.parametrize("m,n,k", [(4400, 4500, 256), (4400, 4500, 384), (8192, 2304, 512)])
-def test_block_gemm_walks_more_tiles_than_compute_units(m, n, k):
+@pytest.mark.parametrize("m,n,k,dtype", [(4400, 4500, 256, torch.bfloat16), (4400, 4500, 384, torch.bfloat16), (8192, 2304, 512, torch.bfloat16),
+                                         (4400, 4500, 256, torch.float16)])
+def test_block_gemm_walks_more_tiles_than_compute_units(m, n, k, dtype):
     """More 256 x 256 tiles than the device has compute units: the large-tile configuration then walks
     several tiles per work-group (even numbers of K steps) and fetches a tile's first slabs during
     the tile before. Ragged last rows and columns; every configuration gives the same bytes."""
     g = torch.Generator().manual_seed(m + k)
-    x = (torch.randn(m, k, generator=g) * torch.logspace(-2, 2, m)[:, None]).to(torch.bfloat16).cuda()
-    w = (torch.randn(n, k, generator=g) * 0.05).to(torch.bfloat16).cuda()
-    bias = (torch.randn(n, generator=g) * 0.1).to(torch.bfloat16).cuda()
+    x = (torch.randn(m, k, generator=g) * torch.logspace(-2, 2, m)[:, None]).to(dtype).cuda()
+    w = (torch.randn(n, k, generator=g) * 0.05).to(dtype).cuda()
+    bias = (torch.randn(n, generator=g) * 0.1).to(dtype).cuda()
     wq, ws = native.quant_blocks(w, "weight")
     xq, xs, xs_t = native.quant_blocks(x, "act", natural=True, kmajor=True)
     cfgs = native.configs(native.KERNEL_GEMM_BLOCKS)
     assert any(c["bm"] * c["bn"] == 256 * 256 for c in cfgs) and (m // 256) * (n // 256) > 256
-    outs = [native.gemm_fp8_blocks(xq, xs_t, wq, ws, bias, torch.bfloat16, c["id"], kmajor=True) for c in cfgs]
+    outs = [native.gemm_fp8_blocks(xq, xs_t, wq, ws, bias, dtype, c["id"], kmajor=True) for c in cfgs]
     torch.cuda.synchronize()
     for c, y in zip(cfgs[1:], outs[1:]):
         assert torch.equal(y, outs[0]), f"configuration {c}"
     # and the same through the natural scale layout, twice in a row (nothing left over between launches)
     for c in cfgs:
         for _ in range(2):
-            assert torch.equal(native.gemm_fp8_blocks(xq, xs, wq, ws, bias, torch.bfloat16, c["id"]), outs[0]), f"configuration {c}"
+            assert torch.equal(native.gemm_fp8_blocks(xq, xs, wq, ws, bias, dtype, c["id"]), outs[0]), f"configuration {c}"
     # rows against the 64-bit product of the dequantized operands
     rows = torch.tensor([0, 255, 256, 2047, m - 1])
     a64 = xq[rows.cuda()].float().double() * xs[rows.cuda()].double().repeat_interleave(128, dim=1)
     w64 = wq.float().double() * ws.double().repeat_interleave(128, dim=0)[:n].repeat_interleave(128, dim=1)
     truth = a64 @ w64.T + bias.double()
-    assert rel_l2(outs[0][rows.cuda()].cpu(), truth.cpu()) <= REL_L2[torch.bfloat16]
+    assert rel_l2(outs[0][rows.cuda()].cpu(), truth.cpu()) <= REL_L2[dtype]
 
 
 def test_block_gemm_uses_every_scale():
