@@ -58,10 +58,13 @@ int64_t km_scales_packed_bytes(int64_t rows, int64_t cols);
 int km_scales_pack(const void *scales, int64_t rows, int64_t cols, void *out, void *stream);
 
 /* Per-tensor e4m3 quantizer: *scale_out = max(amax, 1e-12) / 448 (IEEE division),
- * q = e4m3(clamp(x / scale)). amax_workspace is 4 bytes of device memory the call owns
- * while it runs. Replaces fp8.formats.quantize(x, "tensor")
+ * q = e4m3(clamp(x / scale)). amax_workspace is KM_QUANT_TENSOR_WORKSPACE_BYTES of device memory
+ * (4-byte aligned, contents irrelevant) the call owns while it runs: the abs-max pass leaves one partial
+ * maximum per work-group there and the conversion pass reduces them, so nothing has to be cleared and
+ * no atomics are needed. Replaces fp8.formats.quantize(x, "tensor")
  * (src/kohakumoss_kernels/fp8/formats.py:77-79) and Triton quantize_tensor
  * (backends/triton/fp8/quantize.py:161-168). */
+#define KM_QUANT_TENSOR_WORKSPACE_BYTES 2048
 int km_quant_tensor(const void *x, int64_t rows, int64_t cols, int64_t stride_row, int64_t stride_col,
                     int dtype, void *q, float *scale_out, uint32_t *amax_workspace, void *stream);
 

@@ -338,28 +338,31 @@ __global__ __launch_bounds__(256) void scales_pack(const uint8_t* __restrict__ i
 }
 
 // ---- per-tensor recipe -----------------------------------------------------------------------
-__global__ void fill_u32(uint32_t* p, uint32_t v) { *p = v; }
 
-// The abs-max pass ends in atomics on one address, and those are served one at a time, about 10 ns
-// each, while the wavefronts that issued them keep their slots: 2048 work-groups of 256 threads cost
-// 19 us in atomics on top of 16 us of reading (6144 work-groups: 61 us). So the pass runs few, large
-// work-groups (two per compute unit, 1024 threads, four 128-bit loads in flight per thread), and a
-// work-group first looks at the value with a plain load and skips the atomic when it cannot raise it.
+// The abs-max pass leaves one partial maximum per work-group in the call's workspace and the cast pass
+// reduces them again in every work-group (at most 512 words, from L2, under its first loads): no word
+// to clear beforehand, so no launch for that, and no atomics. Atomics on one address are served one at a
+// time, about 10 ns each, while the wavefronts that issued them keep their slots: 2048 work-groups of 256
+// threads cost 19 us in atomics on top of 16 us of reading; even 512 that first look at the value and skip
+// the atomic when it cannot raise it end in a queue, because they all finish at once. The pass runs few,
+// large work-groups (two per compute unit, 1024 threads, four 128-bit loads in flight per thread and the
+// next four requested before these are looked at).
 // (A single launch that reads the tensor once, keeps it in registers across a grid-wide wait and converts
 // from there was built and measured: 46 us against 44 us for the two passes on [16384, 3072]. Its loads
 // and its stores are separate phases, 32 us even without the wait and the arithmetic, where a streaming
 // kernel overlaps them; the second pass here reads from the last-level cache anyway.)
 constexpr int kAmaxThreads = 1024;
 constexpr int kAmaxBlocks = 512;
+static_assert(kAmaxBlocks * 4 <= KM_QUANT_TENSOR_WORKSPACE_BYTES, "one partial maximum per work-group of the abs-max pass");
 constexpr int kAmaxPiece = kAmaxThreads * 4;  // 128-bit chunks per work-group and trip (64 KiB)
 constexpr int kTensorBlocks = 1 << 20;        // the cast pass: one 16 KiB piece per work-group, grid-stride beyond
 
-// non-negative floats order like their bits: an unsigned atomic max of fp32 bits is an abs-max
-// (NaN patterns stay above infinity)
+// non-negative floats order like their bits: an unsigned max of fp32 bits is an abs-max
+// (NaN patterns stay above infinity). partials[blockIdx.x] = this work-group's maximum.
 template <int DT>
 __global__ __launch_bounds__(kAmaxThreads) void tensor_amax(const uint16_t* __restrict__ x, int64_t sr,
                                                             int64_t sc, int64_t rows, int64_t cols,
-                                                            uint32_t* __restrict__ amax_bits) {
+                                                            uint32_t* __restrict__ partials) {
   constexpr int T = kAmaxThreads;
   const int64_t n = rows * cols;
   const bool dense = sc == 1 && sr == cols;
@@ -368,18 +371,39 @@ __global__ __launch_bounds__(kAmaxThreads) void tensor_amax(const uint16_t* __re
     // a work-group reads whole pieces (four consecutive runs of 16 KiB, one per load of a thread)
     const uint4* src = reinterpret_cast<const uint4*>(x);
     const int64_t nch = n / 8;
-    for (int64_t base = (int64_t)blockIdx.x * kAmaxPiece; base < nch; base += (int64_t)gridDim.x * kAmaxPiece) {
-      const int64_t g = base + threadIdx.x;
-      if (base + kAmaxPiece <= nch) {
-        const uint4 r0 = src[g], r1 = src[g + T], r2 = src[g + 2 * T], r3 = src[g + 3 * T];
-        const uint32_t a = amax16x8(r0), b = amax16x8(r1), c = amax16x8(r2), d = amax16x8(r3);
-        const uint32_t ab = a > b ? a : b, cd = c > d ? c : d, abcd = ab > cd ? ab : cd;
-        m16 = abcd > m16 ? abcd : m16;
-      } else {
-        for (int64_t i = g; i < nch; i += T) {
-          const uint32_t a = amax16x8(src[i]);
-          m16 = a > m16 ? a : m16;
-        }
+    const int64_t first = (int64_t)blockIdx.x * kAmaxPiece, hop = (int64_t)gridDim.x * kAmaxPiece;
+    auto take = [&](const uint4 (&r)[4]) __attribute__((always_inline)) {
+      const uint32_t a = amax16x8(r[0]), b = amax16x8(r[1]), c = amax16x8(r[2]), d = amax16x8(r[3]);
+      const uint32_t ab = a > b ? a : b, cd = c > d ? c : d, abcd = ab > cd ? ab : cd;
+      m16 = abcd > m16 ? abcd : m16;
+    };
+    // whole pieces, the loads of the next one issued before this one is looked at: a work-group that
+    // waits for a piece, reduces it and only then asks for the next leaves the memory system idle in between
+    int64_t base = first;
+    uint4 cur[4], nxt[4];
+    bool have = base + kAmaxPiece <= nch;
+    if (have) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) cur[i] = src[base + threadIdx.x + i * T];
+    }
+    while (have) {
+      const int64_t after = base + hop;
+      const bool more = after + kAmaxPiece <= nch;
+      if (more) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) nxt[i] = src[after + threadIdx.x + i * T];
+      }
+      take(cur);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) cur[i] = nxt[i];
+      base = after;
+      have = more;
+    }
+    // the ragged last piece belongs to the work-group whose walk reaches it
+    if (base < nch) {
+      for (int64_t i = base + threadIdx.x; i < nch; i += T) {
+        const uint32_t a = amax16x8(src[i]);
+        m16 = a > m16 ? a : m16;
       }
     }
   } else {
@@ -397,20 +421,29 @@ __global__ __launch_bounds__(kAmaxThreads) void tensor_amax(const uint16_t* __re
   if (threadIdx.x < 64) {
     const uint32_t mine = threadIdx.x < T / 64 ? wave_m[threadIdx.x] : 0u;
     const uint32_t bits = widen_bits<DT>(wave_max(mine));
-    // the value only ever grows: a (possibly stale) reading at or above this work-group's maximum
-    // means the atomic could not change it
-    if (threadIdx.x == 0 && bits != 0 && bits > __hip_atomic_load(amax_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(amax_bits, bits);
+    if (threadIdx.x == 0) partials[blockIdx.x] = bits;
   }
 }
 
 template <int DT>
 __global__ __launch_bounds__(256) void tensor_cast(const uint16_t* __restrict__ x, int64_t sr,
                                                    int64_t sc, int64_t rows, int64_t cols,
-                                                   const uint32_t* __restrict__ amax_bits,
+                                                   const uint32_t* __restrict__ partials, int npartials,
                                                    uint8_t* __restrict__ q,
                                                    float* __restrict__ scale_out) {
   saturating_conversions();
-  const uint32_t ab = *amax_bits;
+  // the tensor's abs-max: every work-group reduces the abs-max pass's partial maxima (npartials <= 512)
+  __shared__ uint32_t wave_m[4];
+  uint32_t mine = 0;
+  for (int i = threadIdx.x; i < npartials; i += 256) {
+    const uint32_t v = partials[i];
+    mine = v > mine ? v : mine;
+  }
+  mine = wave_max(mine);
+  if ((threadIdx.x & 63) == 0) wave_m[threadIdx.x >> 6] = mine;
+  __syncthreads();
+  const uint32_t ab01 = wave_m[0] > wave_m[1] ? wave_m[0] : wave_m[1], ab23 = wave_m[2] > wave_m[3] ? wave_m[2] : wave_m[3];
+  const uint32_t ab = ab01 > ab23 ? ab01 : ab23;
   const bool finite = ab < kInfBits, nan_all = ab > kInfBits;
   const float s = nan_all ? bits_f32(0x7FC00000u) : __fdiv_rn(bits_f32(ab > kAmaxFloorBits ? ab : kAmaxFloorBits), 448.0f);
   const float rcp = __fdiv_rn(1.0f, s);
@@ -981,7 +1014,6 @@ extern "C" int km_quant_tensor(const void* x, int64_t rows, int64_t cols, int64_
   hipStream_t st = (hipStream_t)stream;
   const int64_t n = rows * cols;
   if (n > 0 && (!x || !q)) return km_fail(KM_ERR_ARG, "km_quant_tensor: null pointer");
-  hipLaunchKernelGGL(fill_u32, dim3(1), dim3(1), 0, st, amax_workspace, 0u);
   int64_t want = (n / 8 + 1023) / 1024;  // one 16 KiB piece per work-group and trip
   unsigned blocks = (unsigned)(want < 1 ? 1 : (want > kTensorBlocks ? kTensorBlocks : want));
   const int64_t amax_want = (n / 8 + kAmaxPiece - 1) / kAmaxPiece;
@@ -989,7 +1021,7 @@ extern "C" int km_quant_tensor(const void* x, int64_t rows, int64_t cols, int64_
   const uint16_t* xp = (const uint16_t*)x;
   KM_DISPATCH_DT(dtype, {
     if (n > 0) hipLaunchKernelGGL(tensor_amax<DT>, dim3(amax_blocks), dim3(kAmaxThreads), 0, st, xp, stride_row, stride_col, rows, cols, amax_workspace);
-    hipLaunchKernelGGL(tensor_cast<DT>, dim3(blocks), dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, amax_workspace, (uint8_t*)q, scale_out);
+    hipLaunchKernelGGL(tensor_cast<DT>, dim3(blocks), dim3(256), 0, st, xp, stride_row, stride_col, rows, cols, amax_workspace, n > 0 ? (int)amax_blocks : 0, (uint8_t*)q, scale_out);
   });
   return km_check_launch("km_quant_tensor");
 }

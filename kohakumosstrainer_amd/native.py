@@ -17,6 +17,7 @@ from torch import Tensor
 LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libkm_kernels.so"
 E4M3 = torch.float8_e4m3fn
 KM_BF16, KM_F16 = 0, 1
+QUANT_TENSOR_WORKSPACE_BYTES = 2048  # KM_QUANT_TENSOR_WORKSPACE_BYTES of include/km_kernels.h
 KM_OK, KM_ERR_ARG, KM_ERR_LAUNCH, KM_ERR_UNSUPPORTED = 0, -1, -2, -3  # return codes of every entry point
 KM_Q_INT8, KM_Q_E4M3 = 0, 1
 KERNEL_GEMM_MX, KERNEL_GEMM_FP8, KERNEL_WO_FWD, KERNEL_WO_DGRAD, KERNEL_GEMM_BLOCKS = 0, 1, 2, 3, 4
@@ -230,7 +231,7 @@ def quant_tensor(x: Tensor) -> tuple[Tensor, Tensor]:
     rows, k = x.shape
     q = torch.empty(rows, k, device=x.device, dtype=torch.uint8)
     s = torch.empty(1, device=x.device, dtype=torch.float32)
-    work = torch.empty(1, device=x.device, dtype=torch.int32)
+    work = torch.empty(QUANT_TENSOR_WORKSPACE_BYTES // 4, device=x.device, dtype=torch.int32)
     with torch.cuda.device(x.device):
         _check(load().km_quant_tensor(x.data_ptr(), rows, k, x.stride(0), x.stride(1), _dtype_code(x.dtype), q.data_ptr(), s.data_ptr(), work.data_ptr(), _stream(x)))
     return q.view(E4M3), s
