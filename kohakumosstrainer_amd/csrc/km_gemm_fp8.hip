@@ -361,7 +361,7 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
     const v4i a_src = pick_rsrc(a_over, na_rsrc, a_rsrc);
     // int8 has no scale to zero the padding step of an odd step count with: its B slab is zeros
     const int b_beyond = I8 ? __builtin_amdgcn_readfirstlane(!b_over && ks + kBAhead >= nk ? (int)0x80000000 : 0) : 0;
-    scale_fetch(s_next, s_over ? nws_base : ws_base, s_over ? nxs_base : xs_base);
+    if constexpr (B3) scale_fetch(s_next, s_over ? nws_base : ws_base, s_over ? nxs_base : xs_base);  // ahead of the B passes, which may stay in flight
     scale_touch(min(ks + 3, nk - 1), b_fill);
     __builtin_amdgcn_sched_barrier(0);
     static_for<TN>([&](auto t_tag) __attribute__((always_inline)) {
@@ -379,6 +379,14 @@ __global__ __launch_bounds__(256, A1 ? 2 : 1) void gemm_fp8_kernel(
       static_for<TM>([&](auto j_tag) __attribute__((always_inline)) {
         constexpr int j = decltype(j_tag)::value;
         constexpr int q = t * TM + j;  // position in the step's MFMA sequence
+        // the scales of the next step are requested behind the step's first MFMA, not ahead of it (the four
+        // wavefronts' loads queue at the address unit, and at the top of the step nothing runs meanwhile);
+        // still ahead of every A pass, so the wait at the step's end covers them
+        if constexpr (q == 1 && !B3) {
+          __builtin_amdgcn_sched_barrier(0);
+          scale_fetch(s_next, s_over ? nws_base : ws_base, s_over ? nxs_base : xs_base);
+          __builtin_amdgcn_sched_barrier(0);
+        }
         if constexpr (I8) {
           // two tiles per pair of slots, low halves then high halves: the two instructions that
           // add into one accumulator are two instructions apart instead of back to back
